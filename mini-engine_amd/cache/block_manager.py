@@ -34,10 +34,12 @@ def hash_block(parent: bytes, token_ids: Seq[int]) -> bytes:
 
 @dataclass(frozen=True)
 class GroupSpec:
-    """One cache group: ``window == 0`` keeps every key; ``window == w`` keeps the last ``w``."""
+    """One cache group: ``window == 0`` keeps every key; ``window == w`` keeps the last ``w`` and, with
+    ``keep_first == f``, the first ``f`` keys of a request as well."""
 
     window: int = 0
     num_blocks: int | None = None  # None: the manager's default
+    keep_first: int = 0
 
 
 class PoolView:
@@ -94,7 +96,7 @@ class BlockManager:
             raise ValueError("at least one cache group is needed")
         self.num_blocks, self.block_size, self.groups = num_blocks, block_size, tuple(groups)
         sizes = [g.num_blocks or num_blocks for g in self.groups]
-        self.core = core or HostCore(block_size, [(g.window, n) for g, n in zip(self.groups, sizes)],
+        self.core = core or HostCore(block_size, [(g.window, n, g.keep_first) for g, n in zip(self.groups, sizes)],
                                      enable_prefix_caching, num_state_slots, has_state)
         self.pools = [PoolView(self.core, g, n) for g, n in enumerate(sizes)]
         self.slots = SlotsView(self.core, num_state_slots) if num_state_slots > 0 else None

@@ -7,7 +7,7 @@ block table per request. A page id indexes every run of its group at once. Each 
 more than the manager hands out: rows that pad a replayed graph write there.
 
 Layout of a layer's pages: keys ``[pages, kv_heads, block_size, head_dim]`` and values transposed,
-``[pages, kv_heads, head_dim, block_size]``, so that the matrix cores read both along the
+``[pages, kv_heads, value_dim, block_size]``, so that the matrix cores read both along the
 contiguous direction (keys along head_dim for q.k, values along the keys for p.v).
 """
 
@@ -50,7 +50,7 @@ def plan_layout(decoder) -> CacheLayout:
             state_layers[i] = need
         elif need is not None:
             raise TypeError(f"layer {i}: unknown cache need {need!r}")
-    groups = [GroupSpec(window=n.window) for n in needs] or [GroupSpec()]
+    groups = [GroupSpec(window=n.window, keep_first=n.keep_first) for n in needs] or [GroupSpec()]
     return CacheLayout(groups, needs, layer_group, state_layers)
 
 
@@ -65,7 +65,7 @@ class CacheStorage:
         for i, g in layout.layer_group.items():
             need = layout.group_needs[g]
             k = torch.zeros((num_blocks + 1, need.num_kv_heads, block_size, need.head_dim), dtype=dtype, device=device)
-            v = torch.zeros((num_blocks + 1, need.num_kv_heads, need.head_dim, block_size), dtype=dtype, device=device)
+            v = torch.zeros((num_blocks + 1, need.num_kv_heads, need.v_dim, block_size), dtype=dtype, device=device)
             self.kv[i] = (k, v)
         for i, need in layout.state_layers.items():
             self.state[i] = torch.zeros((num_state_slots + 1, *need.shape), dtype=need.dtype, device=device)
@@ -79,7 +79,7 @@ class CacheStorage:
     def kv_bytes_per_token(self) -> int:
         """Bytes of keys and values one token occupies over all runs that own pages."""
         elem = torch.empty((), dtype=self.dtype).element_size()
-        return sum(2 * self.layout.group_needs[g].num_kv_heads * self.layout.group_needs[g].head_dim * elem
+        return sum(self.layout.group_needs[g].num_kv_heads * (self.layout.group_needs[g].head_dim + self.layout.group_needs[g].v_dim) * elem
                    for g in self.layout.layer_group.values())
 
     def zero_state(self, slots: list[int]) -> None:

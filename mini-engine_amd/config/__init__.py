@@ -8,11 +8,12 @@ from .registry import (
     read_config_json,
     register_architecture,
 )
-from .specs import AttentionSpec, GatedMlpSpec, LayerSpec, ModelPlan, NormSpec, RotarySpec
+from .specs import AttentionSpec, DecayStateSpec, GatedMlpSpec, LayerSpec, ModelPlan, NormSpec, RotarySpec
 
 __all__ = [
     "ArchitectureEntry",
     "AttentionSpec",
+    "DecayStateSpec",
     "EngineConfig",
     "GatedMlpSpec",
     "LayerSpec",

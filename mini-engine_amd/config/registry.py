@@ -1,6 +1,6 @@
 """One registry from an architecture's name to the functions that describe it.
 
-The name is ``config.json``'s ``architectures[0]``. When that key is absent the ``model_type`` key
+The name is ``config.json``'s ``architectures[0]`` (or its ``architecture``, a string). When that key is absent the ``model_type`` key
 is looked up among the model types that the registered entries claim (the reference keys on
 ``model_type``, ``src/mini_engine/model.py:37``); an entry may also claim configs that name neither
 (``default_for_unnamed``, as the reference takes a config without ``model_type`` for its one model).
@@ -55,6 +55,8 @@ def architecture_name_of(cfg: dict[str, Any]) -> str:
     archs = cfg.get("architectures")
     if archs:
         return str(archs[0])
+    if isinstance(cfg.get("architecture"), str):  # a config that names its one architecture under the singular key
+        return cfg["architecture"]
     model_type = cfg.get("model_type")
     if model_type is None:
         if len(_UNNAMED) != 1:

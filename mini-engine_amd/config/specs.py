@@ -19,23 +19,29 @@ from typing import Any
 
 @dataclass(frozen=True)
 class NormSpec:
-    """Root-mean-square norm over the last ``dim`` elements: ``x * rsqrt(mean(x^2) + eps) * w``."""
+    """Root-mean-square norm over the last ``dim`` elements: ``x * rsqrt(mean(x^2) + eps) * w``. With ``groups > 1``
+    the elements are cut into that many equal consecutive parts, each divided by its own root mean square."""
 
     dim: int
     eps: float
     kind: str = "rmsnorm"
+    groups: int = 1
 
 
 @dataclass(frozen=True)
 class RotarySpec:
-    """Rotate-half rotary position encoding over the first ``rotary_dim`` elements of each head.
+    """Rotary position encoding over the first ``rotary_dim`` elements of each head.
 
-    ``inv_freq[j] = theta ** (-2j / rotary_dim)``; pairs are ``(j, j + rotary_dim/2)``.
+    ``inv_freq[j] = theta ** (-2j / rotary_dim)``; pair ``j`` is ``(j, j + rotary_dim/2)`` with ``pairing ==
+    "halves"`` and ``(2j, 2j + 1)`` with ``"neighbours"``. ``angles == "float64"``: the table of cosines and sines is
+    worked out in double precision before it is rounded to float32 (``"float32"``: angles are float32 products).
     """
 
     rotary_dim: int
     theta: float
     kind: str = "rotary"
+    pairing: str = "halves"
+    angles: str = "float32"
 
 
 @dataclass(frozen=True)
@@ -47,6 +53,11 @@ class AttentionSpec:
     head. ``position`` is ``None`` for a mixer without position encoding. ``cache_from`` names
     another layer (index into ``ModelPlan.layers``) whose keys and values this layer reads instead
     of writing its own.
+
+    ``value_dim``: size of the value heads when it is not ``head_dim``. ``keep_first == f`` (with a window): keys
+    ``0 .. f-1`` stay visible however far the window has moved. ``value_position``: a position encoding over the
+    whole of ``value_dim`` that every value is turned by before it is cached, and every output turned back by at the
+    query's position. ``names`` maps the roles ``q k v o q_norm k_norm`` to the checkpoint's suffixes.
     """
 
     hidden_size: int
@@ -59,11 +70,50 @@ class AttentionSpec:
     position: Any | None = None
     cache_from: int | None = None
     kind: str = "attention"
+    value_dim: int | None = None
+    keep_first: int = 0
+    value_position: Any | None = None
+    names: tuple[tuple[str, str], ...] = ()
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
     @property
     def kv_elements_per_token(self) -> int:
         """Key and value elements one token occupies in this layer's own pages (none when it reads another's)."""
-        return 0 if self.cache_from is not None else 2 * self.num_kv_heads * self.head_dim
+        return 0 if self.cache_from is not None else self.num_kv_heads * (self.head_dim + self.v_dim)
+
+
+@dataclass(frozen=True)
+class DecayStateSpec:
+    """Linear attention with a fixed decay per head and a matrix of state per request and head:
+    ``S_t = decay_h S_(t-1) + k_t v_t^T``, ``o_t = S_t^T q_t`` (no softmax, no denominator).
+
+    ``input_activation`` ("none", "silu") is applied to the q, k and v projections; ``position`` (or None) turns the
+    first elements of q and k; k is multiplied by ``key_scale``. ``output_norm``: "per_head" divides every head's
+    output by its own root mean square (no weight); "all_heads" norms the concatenated heads together, with a weight.
+    The normed outputs are multiplied by ``gate_activation`` ("silu", "sigmoid") of a fourth projection and go through
+    the output projection. ``names`` maps the roles ``q k v g o norm`` to the checkpoint's suffixes.
+    """
+
+    hidden_size: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    decay: tuple[float, ...]
+    norm_eps: float
+    input_activation: str = "none"
+    position: Any | None = None
+    key_scale: float = 1.0
+    output_norm: str = "per_head"
+    gate_activation: str = "silu"
+    names: tuple[tuple[str, str], ...] = ()
+    kind: str = "decay_state"
+
+    @property
+    def state_elements(self) -> int:
+        return self.num_heads * self.key_dim * self.value_dim
 
 
 @dataclass(frozen=True)
@@ -75,6 +125,7 @@ class GatedMlpSpec:
     intermediate_size: int
     activation: str = "silu"
     kind: str = "gated_mlp"
+    names: tuple[tuple[str, str], ...] = ()  # roles ``gate up down`` -> the checkpoint's suffixes
 
 
 @dataclass(frozen=True)
@@ -82,6 +133,8 @@ class LayerSpec:
     """One residual block: which mixer, which feed-forward, which norms, and how they are arranged.
 
     ``arrangement == "pre_norm"``: ``x += mixer(norm1(x)); x += ffn(norm2(x))``.
+    ``arrangement == "parallel"``: ``h = norm1(x); x += residual_scale * (mixer(h) + ffn(h))``: one norm (``mixer_norm``)
+    that both parts read; ``ffn`` may be None (then ``ffn_norm`` and its names are not used).
     The ``*_prefix`` / ``*_name`` strings are the checkpoint names of this layer's tensors.
     """
 
@@ -94,6 +147,7 @@ class LayerSpec:
     mixer_norm_name: str
     ffn_norm_name: str
     arrangement: str = "pre_norm"
+    residual_scale: float = 1.0
 
 
 @dataclass(frozen=True)

@@ -10,7 +10,15 @@
 // ascending order. So the order of every sum depends on p, lo and the head alone, never on how the sequence
 // was cut into steps, on what else is in the batch, or on how many waves share the chunks of a token.
 //
-// Cache layout per layer: keys K[page, kv_head, slot, d]; values transposed V[page, kv_head, d, slot].
+// Cache layout per layer: keys K[page, kv_head, slot, d]; values transposed V[page, kv_head, dv, slot] (dv: the
+// value heads' size, which need not be the keys').
+//
+// Kept first tokens: with keep_first = f > 0 the keys 0 .. f-1 stay visible behind the window. Where the window still
+// reaches them the visible keys are one run from 0; else they are two runs, 0 .. f-1 and lo .. p, and the chunks of the
+// first run (aligned to absolute position like the others) come before those of the second.
+//
+// Values that were turned by their own position before they were cached (pairs of elements, by the angles of a table
+// [positions, 2, dv/2]): the output of a token at position p, a sum of such values, is turned back by p's angles.
 #include "common.h"
 
 #define AG_MAX_D 256
@@ -36,7 +44,8 @@ template <typename T>
 __global__ __launch_bounds__(512) void attention_general_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
-    int table_width, T* __restrict__ out, int num_tokens, int nh, int nkv, int d, int bs, int window, float scale, int wpu) {
+    int table_width, T* __restrict__ out, int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
+    const float* __restrict__ unturn, int un_pairing, float scale, int wpu) {
   constexpr int KMAX = AG_MAX_D / ME_WAVE;
   __shared__ float qs[8][AG_MAX_D];
   __shared__ float parts[8][AG_MAX_D + 2];  // with several waves per unit: a round's results (values, maximum, sum)
@@ -47,7 +56,10 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
   const int t = (int)(unit / nh), head = (int)(unit % nh);
   const int kvh = head / (nh / nkv);
   const int p = positions[t];
-  const int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+  int lo = window > 0 ? (p - window + 1 > 0 ? p - window + 1 : 0) : 0;
+  int kept = keep_first < lo ? keep_first : lo;  // keys 0 .. kept-1 are visible beside lo .. p
+  if (kept == lo) lo = 0, kept = 0;              // the two runs meet: one run from 0
+  const int kept_chunks = (kept + AG_CHUNK - 1) / AG_CHUNK;
   const int* table = block_table + (size_t)token_item[t] * table_width;
 
   const T* qrow = q + ((size_t)t * nh + head) * d;
@@ -62,19 +74,21 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
 
   const bool vec_k = sizeof(T) == 4 && d % 4 == 0 && ((uintptr_t)k_cache & 15) == 0;   // a key row in 16-byte pieces
   const bool vec_v = sizeof(T) == 4 && bs % 4 == 0 && ((uintptr_t)v_cache & 15) == 0;  // four keys of a value row at once
-  const int first_chunk = lo / AG_CHUNK, n_chunks = p / AG_CHUNK - first_chunk + 1;
+  const int first_chunk = lo / AG_CHUNK, n_chunks = kept_chunks + p / AG_CHUNK - first_chunk + 1;
   for (int round = 0; round * wpu < n_chunks; ++round) {
     const int ci = round * wpu + w;  // this wave's chunk of the round, if there is one
     float m = -INFINITY, l = 0.f;
     float acc[KMAX];
 #pragma unroll
     for (int k = 0; k < KMAX; ++k) acc[k] = 0.f;
-    const int chunk0 = (first_chunk + ci) * AG_CHUNK;
-    const int tile_first = ci < n_chunks ? max(chunk0, (lo / 64) * 64) : 1;  // (no chunk left for this wave: no tiles)
-    const int tile_last = ci < n_chunks ? min(p, chunk0 + AG_CHUNK - 1) : 0;
+    const bool of_kept = ci < kept_chunks;  // a chunk of the kept first keys, else of the run lo .. p
+    const int chunk0 = (of_kept ? ci : first_chunk + ci - kept_chunks) * AG_CHUNK;
+    const int vlo = of_kept ? 0 : lo, vhi = of_kept ? kept - 1 : p;  // the run's visible keys
+    const int tile_first = ci < n_chunks ? max(chunk0, (vlo / 64) * 64) : 1;  // (no chunk left for this wave: no tiles)
+    const int tile_last = ci < n_chunks ? min(vhi, chunk0 + AG_CHUNK - 1) : 0;
     for (int tile = tile_first; tile <= tile_last; tile += 64) {
       const int key = tile + lane;
-      const bool valid = key >= lo && key <= p;
+      const bool valid = key >= vlo && key <= vhi;
       float s = -INFINITY;
       if (valid) {
         const int page = table[key / bs];
@@ -109,8 +123,8 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
 #pragma unroll
       for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) acc[k] *= alpha;
       m = m_new;
-      const int j_lo = lo > tile ? lo - tile : 0;
-      const int j_hi = p - tile < 63 ? p - tile : 63;
+      const int j_lo = vlo > tile ? vlo - tile : 0;
+      const int j_hi = vhi - tile < 63 ? vhi - tile : 63;
       int j = j_lo;
       if (vec_v) {
         // whole groups of four keys that lie in one page (tiles and groups are aligned to 4, pages hold a multiple of
@@ -118,11 +132,11 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
         for (; j <= j_hi && (j & 3); ++j) {
           const float pj = __shfl(pr, j, ME_WAVE);
           const int kj = tile + j;
-          const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * d * bs + kj % bs;
+          const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
           for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
             const int i = lane + k * ME_WAVE;
-            if (i < d) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
+            if (i < dv) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
           }
         }
         // eight groups of four keys at a time: their values are requested before the first is used
@@ -133,12 +147,12 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
           for (int gq = 0; gq < 8; ++gq) {
             const bool there = g0 + gq < groups;
             const int kj = tile + j + 4 * (there ? g0 + gq : 0);
-            const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * d * bs + kj % bs;
+            const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
             for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
               const int i = lane + k * ME_WAVE;
               vv[gq][k] = make_float4(0.f, 0.f, 0.f, 0.f);
-              if (there && i < d) vv[gq][k] = *reinterpret_cast<const float4*>(vbase + (size_t)i * bs);
+              if (there && i < dv) vv[gq][k] = *reinterpret_cast<const float4*>(vbase + (size_t)i * bs);
             }
           }
 #pragma unroll
@@ -149,7 +163,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
                           p3 = __shfl(pr, jj + 3, ME_WAVE);
 #pragma unroll
               for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
-                if (lane + k * ME_WAVE < d) {
+                if (lane + k * ME_WAVE < dv) {
                   acc[k] = fmaf(p0, vv[gq][k].x, acc[k]);
                   acc[k] = fmaf(p1, vv[gq][k].y, acc[k]);
                   acc[k] = fmaf(p2, vv[gq][k].z, acc[k]);
@@ -165,11 +179,11 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
         const float pj = __shfl(pr, j, ME_WAVE);
         const int kj = tile + j;
         const int page = table[kj / bs];
-        const T* vbase = v_cache + ((size_t)page * nkv + kvh) * d * bs + kj % bs;
+        const T* vbase = v_cache + ((size_t)page * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
         for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
           const int i = lane + k * ME_WAVE;
-          if (i < d) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
+          if (i < dv) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
         }
       }
     }
@@ -193,12 +207,36 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
     }
   }
   if (w != 0) return;
-  T* orow = out + ((size_t)t * nh + head) * d;
+  T* orow = out + ((size_t)t * nh + head) * dv;
   const float inv = 1.f / lt;
+  if (unturn) {  // the sum of turned values, turned back by this token's angles: through this wave's row of LDS
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int i = lane + k * ME_WAVE;
+      if (i < dv) qw[i] = acct[k] * inv;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS writes of this wave are visible
+    const float* cs = unturn + (size_t)p * dv;  // [2, dv / 2] of this position
+    const int half = dv / 2;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int i = lane + k * ME_WAVE;
+      if (i < dv) {
+        const bool first = un_pairing == 0 ? i < half : (i & 1) == 0;
+        const int j = un_pairing == 0 ? (first ? i : i - half) : i >> 1;
+        const int other = un_pairing == 0 ? (first ? i + half : i - half) : i ^ 1;
+        const float c = cs[j], sn = cs[half + j];
+        orow[i] = from_float<T>(first ? qw[i] * c + qw[other] * sn : qw[i] * c - qw[other] * sn);
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int k = 0; k < KMAX; ++k) {
     const int i = lane + k * ME_WAVE;
-    if (i < d) orow[i] = from_float<T>(acct[k] * inv);
+    if (i < dv) orow[i] = from_float<T>(acct[k] * inv);
   }
 }
 
@@ -404,18 +442,28 @@ __global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
 // `items`: how many items the step's tokens belong to (0: unknown). Steps with two and more tokens per item on
 // average go to the kernel that shares the tiles of keys and values among the tokens of a block; the results are
 // the same bits either way.
-extern "C" int me_attention_general(const void* q, const void* k_cache, const void* v_cache, const int* positions,
-                                    const int* token_item, const int* block_table, int table_width, void* out,
-                                    int num_tokens, int nh, int nkv, int d, int bs, int window, float scale,
-                                    int dtype, int items, hipStream_t stream) {
+//
+// dv: size of the value heads (out is [tokens, nh * dv]); keep_first: the first keys that stay visible behind the window;
+// unturn (float32 [positions, 2, dv/2] or null) and un_pairing (0: element j with j + dv/2; 1: 2j with 2j + 1): the
+// angles that every output row is turned back by. Steps with any of these go to the first kernel.
+extern "C" int me_attention_general_ext(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                                        const int* token_item, const int* block_table, int table_width, void* out,
+                                        int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
+                                        const float* unturn, int un_pairing, float scale, int dtype, int items,
+                                        hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (d <= 0 || d > AG_MAX_D) return me_fail("me_attention_general: head_dim=%d must be in 1..%d", d, AG_MAX_D);
+  if (dv <= 0 || dv > AG_MAX_D) return me_fail("me_attention_general: value head size %d must be in 1..%d", dv, AG_MAX_D);
+  if (keep_first < 0 || (keep_first > 0 && window <= 0))
+    return me_fail("me_attention_general: keep_first=%d needs a window", keep_first);
+  if (unturn && (dv % 2 || (un_pairing & ~1))) return me_fail("me_attention_general: values of size %d, pairing %d", dv, un_pairing);
+  const bool plain = dv == d && keep_first == 0 && !unturn;
   if (nh <= 0 || nkv <= 0 || nh % nkv)
     return me_fail("me_attention_general: %d query heads are not a multiple of %d key/value heads", nh, nkv);
   if (bs <= 0 || table_width <= 0 || window < 0)
     return me_fail("me_attention_general: block_size=%d table_width=%d window=%d", bs, table_width, window);
   const int group = nh / nkv;
-  if (dtype == ME_F32 && items > 0 && num_tokens >= 2 * items && d % 4 == 0 && bs % 4 == 0 && group <= 16 &&
+  if (plain && dtype == ME_F32 && items > 0 && num_tokens >= 2 * items && d % 4 == 0 && bs % 4 == 0 && group <= 16 &&
       (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0) {
     const int tq = 16 / group > 0 ? 16 / group : 1, waves = tq * group;
     const size_t lds = ((size_t)64 * (d + AS_KPAD) + (size_t)d * AS_VROW + (size_t)waves * (d + 64)) * sizeof(float);
@@ -454,10 +502,18 @@ extern "C" int me_attention_general(const void* q, const void* k_cache, const vo
   if (dtype == ME_F32)
     attention_general_kernel<float><<<blocks, waves * 64, 0, stream>>>(
         (const float*)q, (const float*)k_cache, (const float*)v_cache, positions, token_item, block_table,
-        table_width, (float*)out, num_tokens, nh, nkv, d, bs, window, scale, wpu);
+        table_width, (float*)out, num_tokens, nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu);
   else
     attention_general_kernel<bf16_t><<<blocks, waves * 64, 0, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, token_item, block_table,
-        table_width, (bf16_t*)out, num_tokens, nh, nkv, d, bs, window, scale, wpu);
+        table_width, (bf16_t*)out, num_tokens, nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu);
   return me_check_launch("me_attention_general");
+}
+
+extern "C" int me_attention_general(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                                    const int* token_item, const int* block_table, int table_width, void* out,
+                                    int num_tokens, int nh, int nkv, int d, int bs, int window, float scale,
+                                    int dtype, int items, hipStream_t stream) {
+  return me_attention_general_ext(q, k_cache, v_cache, positions, token_item, block_table, table_width, out, num_tokens, nh, nkv,
+                                  d, d, bs, window, 0, nullptr, 0, scale, dtype, items, stream);
 }

@@ -1,0 +1,248 @@
+// Linear attention with a fixed decay per head and a matrix of state per request and head (no softmax, no
+// denominator):
+//
+//   S_t = decay_h * S_(t-1) + k_t v_t^T        (S: [d, dv], float32, kept in a slot between steps)
+//   o_t = S_t^T q_t
+//
+// Three kernels a step. `decay_state_prepare` turns the projections [T, H*d | H*d | H*dv | ...] into float32 q, k
+// and v: an optional activation, an optional rotation of the first rd elements of q and k by the position's angles
+// (either pairing), and a scale on k. `decay_state_scan` walks the new tokens of every item in order, from the state
+// in the item's slot, and leaves the new state there. `decay_state_finish` norms the outputs (every head by its own
+// root mean square, or all heads together with a weight), multiplies by the activation of the gate's projection and
+// rounds to the compute type.
+//
+// Everything from the prepared q, k, v to the normed output is float32, and the scan adds in an order that depends on
+// nothing but the head's sizes: a state column is owned by four lanes of one wave, each walking a quarter of the rows
+// token by token, so a request's outputs are the same bits however its tokens are cut into steps and whatever else the
+// step holds.
+//
+// The decay is carried as two floats (the nearest float and what it misses of the configured value), so that a state
+// that has decayed over thousands of tokens has not drifted by the float's rounding of the decay times its age.
+#include "common.h"
+
+#define DS_MAX_D 256
+
+enum DsAct { DS_ACT_NONE = 0, DS_ACT_SILU = 1, DS_ACT_SIGMOID = 2 };
+
+__device__ __forceinline__ float ds_act(float z, int code) {
+  if (code == DS_ACT_SILU) return z / (1.f + expf(-z));
+  if (code == DS_ACT_SIGMOID) return 1.f / (1.f + expf(-z));
+  return z;
+}
+
+// ---------------------------------------------------------------------------------------------- prepare
+// One wave per (token, head) and kind (q, k, v). Output rows are padded: q32, k32 [T, H, dp] (zeros beyond d),
+// v32 [T, H, dv].
+template <typename T>
+__global__ __launch_bounds__(256) void decay_state_prepare_kernel(
+    const T* __restrict__ proj, int proj_cols, const float* __restrict__ rope_table, int rd, int pairing,
+    const int* __restrict__ positions, float* __restrict__ q32, float* __restrict__ k32, float* __restrict__ v32,
+    int num_tokens, int heads, int d, int dp, int dv, int act, float key_scale) {
+  __shared__ float stage[4][DS_MAX_D];
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const long long unit = (long long)blockIdx.x * 4 + wave;
+  if (unit >= (long long)num_tokens * heads * 3) return;
+  const int kind = (int)(unit % 3), head = (int)((unit / 3) % heads), t = (int)(unit / 3 / heads);
+  const int n = kind == 2 ? dv : d;
+  const T* src = proj + (size_t)t * proj_cols + (kind == 0 ? (size_t)head * d
+                                                 : kind == 1 ? (size_t)heads * d + (size_t)head * d
+                                                             : (size_t)2 * heads * d + (size_t)head * dv);
+  float* st = stage[wave];
+  for (int i = lane; i < n; i += ME_WAVE) st[i] = ds_act(to_float(src[i]), act);
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS writes of this wave are visible
+  if (kind == 2) {
+    float* dst = v32 + ((size_t)t * heads + head) * dv;
+    for (int i = lane; i < dv; i += ME_WAVE) dst[i] = st[i];
+    return;
+  }
+  float* dst = (kind == 0 ? q32 : k32) + ((size_t)t * heads + head) * dp;
+  const float mult = kind == 1 ? key_scale : 1.f;
+  const float* cs = rope_table ? rope_table + (size_t)positions[t] * rd : nullptr;  // [2, rd / 2] of this position
+  const int half = rd / 2;
+  for (int i = lane; i < dp; i += ME_WAVE) {
+    float r = 0.f;
+    if (i < d) {
+      r = st[i];
+      if (cs && i < rd) {
+        const bool first = pairing == 0 ? i < half : (i & 1) == 0;
+        const int j = pairing == 0 ? (first ? i : i - half) : i >> 1;
+        const int other = pairing == 0 ? (first ? i + half : i - half) : i ^ 1;
+        const float c = cs[j], sn = cs[half + j];
+        r = first ? st[i] * c - st[other] * sn : st[i] * c + st[other] * sn;
+      }
+      r *= mult;
+    }
+    dst[i] = r;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------- scan
+// Grid (item, head, 64 columns); a wave owns 16 columns of the state: lane = rg * 16 + column, rg = 0..3 the quarter of
+// the rows (RPL rows a lane, 4 * RPL >= d; q32 and k32 rows are padded to 4 * RPL with zeros). The next token's q, k
+// and v are requested before the current token's arithmetic.
+template <int RPL>
+__global__ __launch_bounds__(256) void decay_state_scan_kernel(
+    const float* __restrict__ q32, const float* __restrict__ k32, const float* __restrict__ v32, float* __restrict__ o32,
+    float* __restrict__ state, const float* __restrict__ decay, const int* __restrict__ item_start,
+    const int* __restrict__ state_slots, int heads, int d, int dv) {
+  constexpr int DP = 4 * RPL;
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const int item = blockIdx.x, head = blockIdx.y;
+  const int col = (blockIdx.z * 4 + wave) * 16 + (lane & 15), rg = lane >> 4;
+  if ((blockIdx.z * 4 + wave) * 16 >= dv) return;  // (whole waves: no block-wide barrier below)
+  const bool has_col = col < dv;
+  const int t0 = item_start[item], t1 = item_start[item + 1];
+  const int slot = state_slots[item];
+  if (slot < 0 || t1 <= t0) return;
+  const float lam = decay[head], lam_lo = decay[heads + head];
+  float* srow = state + (((size_t)slot * heads + head) * d) * dv;  // [d, dv]
+  float S[RPL];
+#pragma unroll
+  for (int r = 0; r < RPL; ++r) {
+    const int i = rg * RPL + r;
+    S[r] = has_col && i < d ? srow[(size_t)i * dv + col] : 0.f;
+  }
+  float4 qn[RPL / 4], kn[RPL / 4];
+  float vn;
+  auto fetch = [&](int t) {
+    const float4* qp = reinterpret_cast<const float4*>(q32 + ((size_t)t * heads + head) * DP + rg * RPL);
+    const float4* kp = reinterpret_cast<const float4*>(k32 + ((size_t)t * heads + head) * DP + rg * RPL);
+#pragma unroll
+    for (int r = 0; r < RPL / 4; ++r) qn[r] = qp[r], kn[r] = kp[r];
+    vn = has_col ? v32[((size_t)t * heads + head) * dv + col] : 0.f;
+  };
+  fetch(t0);
+  for (int t = t0; t < t1; ++t) {
+    float4 qc[RPL / 4], kc[RPL / 4];
+#pragma unroll
+    for (int r = 0; r < RPL / 4; ++r) qc[r] = qn[r], kc[r] = kn[r];
+    const float vc = vn;
+    if (t + 1 < t1) fetch(t + 1);
+    float o = 0.f;
+#pragma unroll
+    for (int r = 0; r < RPL / 4; ++r) {
+      const float kk[4] = {kc[r].x, kc[r].y, kc[r].z, kc[r].w};
+      const float qq[4] = {qc[r].x, qc[r].y, qc[r].z, qc[r].w};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float s = S[4 * r + u];
+        const float sn = fmaf(lam_lo, s, fmaf(lam, s, kk[u] * vc));
+        S[4 * r + u] = sn;
+        o = fmaf(sn, qq[u], o);
+      }
+    }
+    o += __shfl_xor(o, 16, ME_WAVE);
+    o += __shfl_xor(o, 32, ME_WAVE);
+    if (rg == 0 && has_col) o32[((size_t)t * heads + head) * dv + col] = o;
+  }
+#pragma unroll
+  for (int r = 0; r < RPL; ++r) {
+    const int i = rg * RPL + r;
+    if (has_col && i < d) srow[(size_t)i * dv + col] = S[r];
+  }
+}
+
+// ----------------------------------------------------------------------------------------------- finish
+// One block per token. norm_kind 0: every head's dv outputs over their own sqrt(mean^2 + eps), no weight;
+// 1: all heads' outputs together over sqrt(mean^2 + eps), times w [heads * dv]. Then times act(gate), where the gate
+// is the last heads * dv columns of the projections.
+template <typename T>
+__global__ __launch_bounds__(256) void decay_state_finish_kernel(const float* __restrict__ o32, const T* __restrict__ proj,
+                                                                  int proj_cols, int gate_at, const float* __restrict__ w,
+                                                                  T* __restrict__ out, int heads, int dv, int norm_kind,
+                                                                  int gate_act, float eps) {
+  __shared__ float inv[DS_MAX_D];  // per head (norm_kind 0: at most DS_MAX_D heads), or one value
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1), waves = blockDim.x / ME_WAVE;
+  const int t = blockIdx.x, n = heads * dv;
+  const float* orow = o32 + (size_t)t * n;
+  if (norm_kind == 0) {
+    for (int h = wave; h < heads; h += waves) {
+      float ss = 0.f;
+      for (int i = lane; i < dv; i += ME_WAVE) ss = fmaf(orow[h * dv + i], orow[h * dv + i], ss);
+      ss = wave_sum(ss);
+      if (lane == 0) inv[h] = rsqrtf(ss / (float)dv + eps);
+    }
+  } else {  // a wave adds up the whole row: the order follows from its length alone
+    if (wave == 0) {
+      float ss = 0.f;
+      for (int i = lane; i < n; i += ME_WAVE) ss = fmaf(orow[i], orow[i], ss);
+      ss = wave_sum(ss);
+      if (lane == 0) inv[0] = rsqrtf(ss / (float)n + eps);
+    }
+  }
+  __syncthreads();
+  const T* gate = proj + (size_t)t * proj_cols + gate_at;
+  T* dst = out + (size_t)t * n;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    float y = orow[i] * (norm_kind == 0 ? inv[i / dv] : inv[0] * w[i]);
+    y *= ds_act(to_float(gate[i]), gate_act);
+    dst[i] = from_float<T>(y);
+  }
+}
+
+// --------------------------------------------------------------------------------------------- entry points
+extern "C" int me_decay_state_padded_dim(int d) {  // the row length of the prepared q and k
+  return d <= 32 ? 32 : d <= 64 ? 64 : d <= 128 ? 128 : 256;
+}
+
+// Bytes of float32 workspace that a step of `tokens` tokens needs (prepared q, k, v and the raw outputs).
+extern "C" long long me_decay_state_workspace(long long tokens, int heads, int d, int dv) {
+  const long long dp = me_decay_state_padded_dim(d);
+  return tokens * heads * (2 * dp + 2 * (long long)dv) * 4 + 1024;
+}
+
+// proj [T, proj_cols]: q heads, k heads (d each), v heads, gate (dv each), so proj_cols = 2 heads (d + dv).
+// decay: float32 [2, heads] (the decay's nearest float, then the rest of the configured value).
+// state: float32 [slots, heads, d, dv]; item_start [items + 1], state_slots [items] (a negative slot: the item is skipped).
+extern "C" int me_decay_state(const void* proj, const float* rope_table, int rd, int pairing, const int* positions,
+                              const float* decay, const float* norm_w, float* state, const int* item_start,
+                              const int* state_slots, void* out, void* workspace, int num_tokens, int items, int heads, int d,
+                              int dv, int in_act, float key_scale, int norm_kind, int gate_act, float eps, int dtype,
+                              hipStream_t stream) {
+  if (num_tokens <= 0 || items <= 0) return 0;
+  if (heads <= 0 || heads > DS_MAX_D || d <= 0 || d > DS_MAX_D || dv <= 0)
+    return me_fail("me_decay_state: heads=%d d=%d dv=%d (heads and key size up to %d)", heads, d, dv, DS_MAX_D);
+  if (rope_table && (rd <= 0 || rd > d || rd % 2 || (pairing & ~1)))
+    return me_fail("me_decay_state: rotary_dim=%d with head size %d, pairing %d", rd, d, pairing);
+  if (norm_kind != 0 && norm_kind != 1) return me_fail("me_decay_state: norm kind %d", norm_kind);
+  if (norm_kind == 1 && !norm_w) return me_fail("me_decay_state: the norm over all heads needs its weight");
+  if (items > 65535 * 16 || heads > 65535) return me_fail("me_decay_state: %d items, %d heads", items, heads);
+  if ((uintptr_t)workspace & 15) return me_fail("me_decay_state: the workspace must be aligned to 16 bytes");
+  const int dp = me_decay_state_padded_dim(d);
+  const int proj_cols = 2 * heads * (d + dv);
+  float* q32 = (float*)workspace;
+  float* k32 = q32 + (size_t)num_tokens * heads * dp;
+  float* v32 = k32 + (size_t)num_tokens * heads * dp;
+  float* o32 = v32 + (size_t)num_tokens * heads * dv;
+  const long long units = (long long)num_tokens * heads * 3;
+  const unsigned prep_blocks = (unsigned)((units + 3) / 4);
+  const dim3 scan_grid(items, heads, (dv + 63) / 64);
+  if (scan_grid.z > 65535) return me_fail("me_decay_state: value heads of %d elements", dv);
+#define DS_SCAN(RPL)                                                                                                        \
+  decay_state_scan_kernel<RPL><<<scan_grid, 256, 0, stream>>>(q32, k32, v32, o32, state, decay, item_start, state_slots, heads, \
+                                                              d, dv)
+#define DS_RUN(T)                                                                                                           \
+  do {                                                                                                                      \
+    decay_state_prepare_kernel<T><<<prep_blocks, 256, 0, stream>>>((const T*)proj, proj_cols, rope_table, rd, pairing,        \
+                                                                   positions, q32, k32, v32, num_tokens, heads, d, dp, dv,   \
+                                                                   in_act, key_scale);                                       \
+    if (dp == 32)                                                                                                           \
+      DS_SCAN(8);                                                                                                           \
+    else if (dp == 64)                                                                                                      \
+      DS_SCAN(16);                                                                                                          \
+    else if (dp == 128)                                                                                                     \
+      DS_SCAN(32);                                                                                                          \
+    else                                                                                                                    \
+      DS_SCAN(64);                                                                                                          \
+    decay_state_finish_kernel<T><<<num_tokens, 256, 0, stream>>>(o32, (const T*)proj, proj_cols, 2 * heads * d + heads * dv, \
+                                                                 norm_w, (T*)out, heads, dv, norm_kind, gate_act, eps);      \
+  } while (0)
+  if (dtype == ME_F32)
+    DS_RUN(float);
+  else
+    DS_RUN(bf16_t);
+#undef DS_RUN
+#undef DS_SCAN
+  return me_check_launch("me_decay_state");
+}

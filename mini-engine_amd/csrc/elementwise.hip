@@ -737,3 +737,244 @@ extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const 
                               write_kv, wide, tiles, hpb, grid, item_start, num_items, num_segments, stream);
   return me_check_launch("me_qk_norm_rope_scatter");
 }
+
+// ------------------------------------------------- residual add (scaled) + RMS norm in groups
+// For output row r (input row src = rows ? rows[r] : r):
+//   s = x[src] + delta_scale * (delta[src] + sum of the partial sums);  if (write_x) x[src] = s;
+//   the row is cut into `groups` equal consecutive parts, each divided by its own sqrt(mean(part^2) + eps);
+//   h[r] = that, times w.
+// One block per row, a wave per group at a time: a group's sum of squares is added up in an order that its length
+// alone fixes. groups == 1 and delta_scale == 1 is the norm of the kernels above.
+#define ME_MAX_NORM_GROUPS 64
+
+template <typename T>
+__global__ void add_group_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ parts,
+                                         int num_parts, size_t part_stride, float delta_scale, const float* __restrict__ w,
+                                         T* __restrict__ h, const int* __restrict__ rows, int dim, int groups, float eps,
+                                         int write_x) {
+  __shared__ float inv[ME_MAX_NORM_GROUPS];
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1), waves = blockDim.x / ME_WAVE;
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* xr = x + (size_t)src * dim;
+  const T* dr = delta ? delta + (size_t)src * dim : nullptr;
+  const float* pr = parts ? parts + (size_t)src * dim : nullptr;
+  const bool adds = dr || pr;
+  const int gs = dim / groups;
+  auto sum_at = [&](int i) {
+    float d = 0.f;
+    if (dr) d = to_float(dr[i]);
+    if (pr) {
+      float q = pr[i];
+      for (int p = 1; p < num_parts; ++p) q += pr[p * part_stride + i];
+      d += q;
+    }
+    return adds ? fmaf(delta_scale, d, xr[i]) : xr[i];
+  };
+  for (int g = wave; g < groups; g += waves) {
+    float ss = 0.f;
+    for (int i = g * gs + lane; i < (g + 1) * gs; i += ME_WAVE) {
+      const float s = sum_at(i);
+      if (write_x && adds) xr[i] = s;
+      ss = fmaf(s, s, ss);
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) inv[g] = rsqrtf(ss / (float)gs + eps);
+  }
+  __syncthreads();
+  T* hr = h + (size_t)r * dim;
+  for (int i = threadIdx.x; i < dim; i += blockDim.x) {
+    const float s = (adds && !write_x) ? sum_at(i) : xr[i];
+    hr[i] = from_float<T>(s * inv[i / gs] * w[i]);
+  }
+}
+
+extern "C" int me_add_group_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride,
+                                    float delta_scale, const float* w, void* h, const int* rows, int num_rows, int dim,
+                                    int groups, float eps, int write_x, int dtype, hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  if (dim <= 0 || groups < 1 || groups > ME_MAX_NORM_GROUPS || dim % groups)
+    return me_fail("me_add_group_rmsnorm: dim=%d in %d groups (1..%d equal parts)", dim, groups, ME_MAX_NORM_GROUPS);
+  if (parts && (num_parts < 1 || part_stride < (long long)dim)) return me_fail("me_add_group_rmsnorm: %d partial sums", num_parts);
+  const int threads = dim >= 1024 ? 256 : (dim >= 256 ? 128 : 64);
+  if (dtype == ME_F32)
+    add_group_rmsnorm_kernel<float><<<num_rows, threads, 0, stream>>>((float*)x, (const float*)delta, parts, num_parts,
+                                                                      (size_t)part_stride, delta_scale, w, (float*)h, rows, dim,
+                                                                      groups, eps, write_x);
+  else
+    add_group_rmsnorm_kernel<bf16_t><<<num_rows, threads, 0, stream>>>((float*)x, (const bf16_t*)delta, parts, num_parts,
+                                                                       (size_t)part_stride, delta_scale, w, (bf16_t*)h, rows,
+                                                                       dim, groups, eps, write_x);
+  return me_check_launch("me_add_group_rmsnorm");
+}
+
+// x += scale * (delta + the partial sums, in the order of the runs): the residual add of a block that multiplies
+// what its parts give.
+template <typename T>
+__global__ void residual_add_scaled_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ parts,
+                                           int num_parts, size_t part_stride, float scale, size_t count) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x) {
+    float d = 0.f;
+    if (delta) d = to_float(delta[i]);
+    if (parts) {
+      float q = parts[i];
+      for (int p = 1; p < num_parts; ++p) q += parts[p * part_stride + i];
+      d += q;
+    }
+    x[i] = fmaf(scale, d, x[i]);
+  }
+}
+
+extern "C" int me_residual_add_scaled(void* x, const void* delta, const float* parts, int num_parts, long long part_stride,
+                                      float scale, int num_rows, int dim, int dtype, hipStream_t stream) {
+  if (num_rows <= 0 || dim <= 0) return 0;
+  if (!delta && !parts) return 0;
+  if (parts && num_parts < 1) return me_fail("me_residual_add_scaled: partial sums without parts");
+  const size_t count = (size_t)num_rows * dim;
+  const size_t want = (count + 255) / 256;
+  const int blocks = (int)(want < 4096 ? want : 4096);
+  if (dtype == ME_F32)
+    residual_add_scaled_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, (const float*)delta, parts, num_parts,
+                                                                  (size_t)part_stride, scale, count);
+  else
+    residual_add_scaled_kernel<bf16_t><<<blocks, 256, 0, stream>>>((float*)x, (const bf16_t*)delta, parts, num_parts,
+                                                                   (size_t)part_stride, scale, count);
+  return me_check_launch("me_residual_add_scaled");
+}
+
+// ------------------------------------- q/k norm + rotation in either pairing + rotated values + page write
+// qkv is [T, nh * d + nkv * d + nkv * dv]: query heads, key heads of size d, then value heads of size dv.
+// A wave per head at a time:
+//   q, k heads: optional RMS norm over d with q_w / k_w, then the first rd elements turned by the position's angles
+//               (pairing 0: element j with j + rd/2; pairing 1: element 2j with 2j + 1), the rest unchanged;
+//   v heads:    with v_table, all dv elements turned by the position's angles of that table, in v_pairing; else copied.
+// q goes to q_out [T, nh, d], keys to K[page, kvh, slot, d], values to V[page, kvh, dv, slot].
+// Tables are float32 [positions, 2, n/2] (cosines, then sines) for n = rd and n = dv.
+__device__ __forceinline__ void pair_of(int i, int n, int pairing, int& j, int& other, bool& first) {
+  if (pairing == 0) {
+    const int half = n / 2;
+    first = i < half;
+    j = first ? i : i - half;
+    other = first ? i + half : i - half;
+  } else {
+    first = (i & 1) == 0;
+    j = i >> 1;
+    other = i ^ 1;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_rotate_scatter_kernel(
+    const T* __restrict__ qkv, const float* __restrict__ q_w, const float* __restrict__ k_w,
+    const float* __restrict__ rope_table, int rd, int pairing, const float* __restrict__ v_table, int v_pairing,
+    const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
+    int table_width, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int nkv, int d, int dv,
+    int bs, float eps, int heads_per_block) {
+  __shared__ float stage[4][ME_MAX_HEAD_DIM];
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const int t = blockIdx.x;
+  const int heads_total = nh + 2 * nkv;
+  const size_t width = (size_t)(nh + nkv) * d + (size_t)nkv * dv;
+  const int pos = positions[t];
+  const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
+  const int hd_end = min(heads_total, (int)(blockIdx.y + 1) * heads_per_block);
+  for (int hd = blockIdx.y * heads_per_block + wave; hd < hd_end; hd += 4) {
+    const int kind = hd < nh ? 0 : (hd < nh + nkv ? 1 : 2);
+    const int n = kind == 2 ? dv : d;
+    const T* src = qkv + (size_t)t * width + (kind == 2 ? (size_t)(nh + nkv) * d + (size_t)(hd - nh - nkv) * dv : (size_t)hd * d);
+    float vals[ME_MAX_HEAD_DIM / ME_WAVE];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+      const int i = lane + k * ME_WAVE;
+      vals[k] = i < n ? to_float(src[i]) : 0.f;
+      ss = fmaf(vals[k], vals[k], ss);
+    }
+    const float* w = kind == 0 ? q_w : (kind == 1 ? k_w : nullptr);
+    if (w) {
+      const float inv = rsqrtf(wave_sum(ss) / (float)d + eps);
+#pragma unroll
+      for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (i < d) vals[k] = vals[k] * inv * w[i];
+      }
+    }
+    const float* table = kind == 2 ? v_table : rope_table;
+    const int turn = kind == 2 ? dv : rd, how = kind == 2 ? v_pairing : pairing;
+    if (table && turn > 0) {
+      const float* cs = table + (size_t)pos * turn;  // [2, turn / 2] of this position
+      float* st = stage[wave];
+      __builtin_amdgcn_wave_barrier();  // the previous head's reads of this wave's stage are done
+#pragma unroll
+      for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (i < n) st[i] = vals[k];
+      }
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): LDS writes of this wave are visible
+#pragma unroll
+      for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (i < turn) {
+          int j, other;
+          bool first;
+          pair_of(i, turn, how, j, other, first);
+          const float c = cs[j], sn = cs[turn / 2 + j];
+          vals[k] = first ? st[i] * c - st[other] * sn : st[i] * c + st[other] * sn;
+        }
+      }
+    }
+    if (kind == 0) {
+      T* dst = q_out + ((size_t)t * nh + hd) * d;
+#pragma unroll
+      for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+        const int i = lane + k * ME_WAVE;
+        if (i < d) dst[i] = from_float<T>(vals[k]);
+      }
+    } else if (page >= 0) {
+      if (kind == 1) {
+        T* dst = k_cache + (((size_t)page * nkv + (hd - nh)) * bs + slot) * d;
+#pragma unroll
+        for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+          const int i = lane + k * ME_WAVE;
+          if (i < d) dst[i] = from_float<T>(vals[k]);
+        }
+      } else {
+        T* dst = v_cache + ((size_t)page * nkv + (hd - nh - nkv)) * dv * bs + slot;
+#pragma unroll
+        for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
+          const int i = lane + k * ME_WAVE;
+          if (i < dv) dst[(size_t)i * bs] = from_float<T>(vals[k]);
+        }
+      }
+    }
+  }
+}
+
+extern "C" int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd,
+                                     int pairing, const float* v_table, int v_pairing, const int* positions,
+                                     const int* token_item, const int* block_table, int table_width, void* q_out,
+                                     void* k_cache, void* v_cache, int num_tokens, int nh, int nkv, int d, int dv, int bs,
+                                     float eps, int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (d <= 0 || d > ME_MAX_HEAD_DIM || dv <= 0 || dv > ME_MAX_HEAD_DIM)
+    return me_fail("me_qkv_rotate_scatter: head sizes %d and %d must be in 1..%d", d, dv, ME_MAX_HEAD_DIM);
+  if (rope_table && (rd <= 0 || rd > d || rd % 2)) return me_fail("me_qkv_rotate_scatter: rotary_dim=%d with head_dim=%d", rd, d);
+  if (v_table && dv % 2) return me_fail("me_qkv_rotate_scatter: values of odd size %d cannot be turned in pairs", dv);
+  if ((pairing | v_pairing) & ~1) return me_fail("me_qkv_rotate_scatter: pairing is 0 (halves) or 1 (neighbours)");
+  if (nh <= 0 || nkv <= 0 || bs <= 0 || table_width <= 0)
+    return me_fail("me_qkv_rotate_scatter: nh=%d nkv=%d block_size=%d table_width=%d", nh, nkv, bs, table_width);
+  const int heads_total = nh + 2 * nkv;
+  const int hpb = num_tokens >= 512 ? heads_total : 4;
+  dim3 grid(num_tokens, (heads_total + hpb - 1) / hpb);
+  if (grid.y > 65535) return me_fail("me_qkv_rotate_scatter: too many heads");
+  if (dtype == ME_F32)
+    qkv_rotate_scatter_kernel<float><<<grid, 256, 0, stream>>>(
+        (const float*)qkv, q_w, k_w, rope_table, rd, pairing, v_table, v_pairing, positions, token_item, block_table, table_width,
+        (float*)q_out, (float*)k_cache, (float*)v_cache, nh, nkv, d, dv, bs, eps, hpb);
+  else
+    qkv_rotate_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+        (const bf16_t*)qkv, q_w, k_w, rope_table, rd, pairing, v_table, v_pairing, positions, token_item, block_table, table_width,
+        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, dv, bs, eps, hpb);
+  return me_check_launch("me_qkv_rotate_scatter");
+}

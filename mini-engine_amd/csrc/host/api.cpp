@@ -56,7 +56,7 @@ extern "C" {
 int me_host_error_kind() { return g_kind; }
 
 // settings: block_size, prefix_caching, num_state_slots, has_state, max_num_seqs, max_num_batched_tokens,
-// max_model_len; groups: (window, num_pages) per cache group.
+// max_model_len; groups: (window, num_pages, keep_first) per cache group.
 void* me_core_new(const int32_t* settings, const int32_t* groups, int num_groups, const int32_t* eos, int num_eos,
                   uint64_t seed) {
   try {
@@ -69,7 +69,7 @@ void* me_core_new(const int32_t* settings, const int32_t* groups, int num_groups
     c.max_num_seqs = settings[4];
     c.max_num_batched_tokens = settings[5];
     c.max_model_len = settings[6];
-    for (int g = 0; g < num_groups; ++g) c.groups.push_back({groups[2 * g], groups[2 * g + 1]});
+    for (int g = 0; g < num_groups; ++g) c.groups.push_back({groups[3 * g], groups[3 * g + 1], groups[3 * g + 2]});
     c.eos_ids.assign(eos, eos + num_eos);
     c.seed = seed;
     return new CoreBox(c);

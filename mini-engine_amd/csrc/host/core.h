@@ -129,6 +129,7 @@ struct Request {
 struct GroupConfig {
   int window = 0;  // 0: every key stays needed; w: a query sees the last w keys
   int num_pages = 0;
+  int keep_first = 0;  // with a window: the first keys of a request stay needed however far the window has moved
 };
 
 struct CoreConfig {

@@ -142,6 +142,8 @@ Core::Core(const CoreConfig& config) : config_(config) {
   for (const GroupConfig& g : config_.groups) {
     if (g.num_pages < 1) throw Error(kBadValue, "num_blocks must be positive");
     if (g.window < 0) throw Error(kBadValue, "a window must be >= 0");
+    if (g.keep_first < 0 || (g.keep_first > 0 && g.window == 0))
+      throw Error(kBadValue, "kept first keys must be >= 0 and need a window");
     pools_.emplace_back(g.num_pages);
     all_kept = all_kept && g.window == 0;
   }
@@ -165,13 +167,14 @@ long Core::evictions() const {
 
 // Whether a request of this many tokens could hold what a step of it needs, all pools empty. A group
 // that keeps every key needs all of the request's pages; a window group needs the window and the
-// longest portion a step may bring, plus a page for the portion's ragged start.
+// longest portion a step may bring, plus a page for the portion's ragged start, plus the pages of the first keys it keeps.
 bool Core::can_ever_hold(int tokens) const {
   const int all = blocks_for(tokens);
   for (size_t g = 0; g < pools_.size(); ++g) {
     int need = all;
     const int w = config_.groups[g].window;
-    if (w > 0) need = std::min(all, blocks_for(w + std::min(config_.max_num_batched_tokens, tokens)) + 1);
+    if (w > 0)
+      need = std::min(all, blocks_for(w + std::min(config_.max_num_batched_tokens, tokens)) + 1 + blocks_for(config_.groups[g].keep_first));
     if (need > pools_[g].num_pages()) return false;
   }
   return true;
@@ -263,7 +266,7 @@ void Core::drop(Request* r) {
 }
 
 // Pages of window groups that no later query of `r` can see go back at once: a query at position
-// p >= num_computed sees the keys from p - window + 1 on.
+// p >= num_computed sees the keys from p - window + 1 on, and the group's kept first keys, whose pages stay.
 int Core::drop_passed(Request* r) {
   int freed = 0;
   for (size_t g = 0; g < r->tables.size() && g < pools_.size(); ++g) {
@@ -272,7 +275,7 @@ int Core::drop_passed(Request* r) {
     const int first_needed = std::max(0, r->num_computed - w + 1);
     std::vector<int32_t>& table = r->tables[g];
     const int whole = std::min((int)table.size(), first_needed / config_.block_size);
-    for (int i = 0; i < whole; ++i)
+    for (int i = blocks_for(config_.groups[g].keep_first); i < whole; ++i)
       if (table[i] >= 0) {
         pools_[g].release(table[i]);
         table[i] = -1;

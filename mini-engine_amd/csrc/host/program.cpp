@@ -47,6 +47,7 @@ struct Pending {
   const float* ss = nullptr;
   int ss_blocks = 0;
   const void* carried_w = nullptr;
+  float scale = 1.f;  // what the block multiplies the delta by when it is added to the stream
   bool any() const { return delta || parts; }
   bool carried() const { return ss != nullptr; }
 };
@@ -136,6 +137,15 @@ SplitPlan split_plan(int items, int kv_units, int max_ctx, int least_live, const
   return {keys, splits, std::min(full, splits), live_count};
 }
 
+// An attention operation that the kernels of the plain form serve: keys and values of one size, a window without kept
+// first keys, rotation of halves, values as they are.
+bool attention_is_plain(const Op& op) {
+  return (op.i[9] == 0 || op.i[9] == op.i[2]) && op.i[10] == 0 && op.i[11] == 0 && op.i[12] == 0;
+}
+
+int groups_of(int64_t v) { return v > 1 ? (int)v : 1; }
+float scale_of(float f) { return f == 0.f ? 1.f : f; }
+
 class Run {
  public:
   Run(const Program& prog, const std::vector<Value>& values, const StepView& s, Arena& arena, int32_t* fed_tokens,
@@ -185,7 +195,7 @@ class Run {
         norm_linear(op);
         break;
       case kOpNorm:
-        add_norm((const float*)op.p[0], op.f[0], bufs_[op.out]);
+        add_norm((const float*)op.p[0], op.f[0], bufs_[op.out], groups_of(op.i[0]));
         break;
       case kOpLinear:
         product(bufs_[op.in], op.p[1], (int)op.i[0], (int)op.i[1], (int)op.i[2], dtype_, bufs_[op.out]);
@@ -196,6 +206,10 @@ class Run {
       case kOpDelta:
         pending_ = Pending();
         pending_.delta = bufs_[op.in];
+        pending_.scale = scale_of(op.f[0]);
+        break;
+      case kOpDecayState:
+        decay_state(op);
         break;
       case kOpAttention:
         attention(op);
@@ -207,7 +221,10 @@ class Run {
         sample();
         break;
       case kOpAdd:
-        if (pending_.any())
+        if (pending_.any() && pending_.scale != 1.f)
+          ok(me_residual_add_scaled(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, pending_.scale, t_, h_,
+                                    dtype_, stream_));
+        else if (pending_.any())
           ok(me_residual_add(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, t_, h_, dtype_, stream_));
         pending_ = Pending();
         release_parts();
@@ -224,9 +241,13 @@ class Run {
   }
 
   // x += pending; out = rmsnorm(x) * w, as a kernel of its own.
-  void add_norm(const float* w, float eps, void* out) {
-    ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, w, out, nullptr, t_, h_, eps, 1,
-                      dtype_, stream_));
+  void add_norm(const float* w, float eps, void* out, int groups = 1) {
+    if (groups > 1 || pending_.scale != 1.f)  // a norm in groups, or a block that multiplies what its parts give
+      ok(me_add_group_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, pending_.scale, w, out,
+                              nullptr, t_, h_, groups, eps, 1, dtype_, stream_));
+    else
+      ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, w, out, nullptr, t_, h_, eps, 1,
+                        dtype_, stream_));
     pending_ = Pending();
     release_parts();
   }
@@ -257,6 +278,11 @@ class Run {
         throw Error(kBroken, "a norm was left to a product whose kernel does not scale its rows");
       pending_ = Pending();
       release_parts();
+      return;
+    }
+    if (groups_of(op.i[3]) > 1 || pending_.scale != 1.f) {  // no product of this folder carries such a norm as its prologue
+      add_norm(w_norm, op.f[0], normed_, groups_of(op.i[3]));
+      product(normed_, op.p[1], rows_of_w, k, gated, dtype_, bufs_[op.out]);
       return;
     }
     const int pending = pending_.parts ? kPendingParts : pending_.delta ? kPendingTensor : kPendingNone;
@@ -322,7 +348,9 @@ class Run {
     const int n = (int)op.i[0], k = (int)op.i[1];
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
+    const float scale = scale_of(op.f[0]);
     pending_ = Pending();
+    pending_.scale = scale;
     if (attn_parts_.o) {  // decode attention left its splits to this product
       const AttnParts a = attn_parts_;
       attn_parts_ = AttnParts();
@@ -336,7 +364,7 @@ class Run {
       pending_.stride = (long long)t_ * n;
       return;
     }
-    if (next_ && next_->kind == kOpNormLinear && next_->i[1] == h_ &&
+    if (scale == 1.f && next_ && next_->kind == kOpNormLinear && next_->i[1] == h_ && groups_of(next_->i[3]) == 1 &&
         choose_carried_norm(dtype_, t_, n, k, (int)next_->i[0], (int)next_->i[2], compute_units(), true)) {
       // x += product in the product's epilogue, which also starts the norm behind it (choice.cpp)
       const int blocks = me_gemm_bf16_stream_carry_blocks(t_, n, k, compute_units());
@@ -350,7 +378,10 @@ class Run {
     }
     const ProductChoice c = choose_product(dtype_, kRoleDeltaInto, t_, n, k, 0, dtype_, compute_units(), true);
     if (c.adds_into) {  // x += product, in the library's epilogue: nothing stays pending
-      if (library_adds(x, op.p[1], x_, t_, n, k, stream_)) return;
+      if (scale == 1.f && library_adds(x, op.p[1], x_, t_, n, k, stream_)) {
+        pending_ = Pending();
+        return;
+      }
       // (a size the library has no algorithm for: the product as one partial sum, through this folder's kernels)
       parts_mark_ = arena_.used;
       float* sum = (float*)arena_.take((size_t)t_ * n * 4);
@@ -392,6 +423,18 @@ class Run {
                                  std::to_string(s_.max_ctx));
     void* out = bufs_[op.out];
     const void* qkv = bufs_[op.in];
+    if (!attention_is_plain(op)) {  // value heads of their own size, kept first keys, the other pairing, turned values
+      const int dv = op.i[9] ? (int)op.i[9] : d, keep_first = (int)op.i[10], pairing = (int)op.i[11];
+      const float* v_table = op.i[12] ? (const float*)op.p[5] : nullptr;
+      const int v_pairing = op.i[12] ? (int)op.i[12] - 1 : 0;
+      if (!owns) throw Error(kBadValue, "an attention layer of this form writes its own pages");
+      void* q = arena_.take((size_t)t_ * nh * d * elem_);
+      ok(me_qkv_rotate_scatter(qkv, q_w, k_w, rope, rd, pairing, v_table, v_pairing, idx(s_.lay.positions), idx(s_.lay.token_item),
+                               table, width, q, kc, vc, t_, nh, nkv, d, dv, bs, eps, dtype_, stream_));
+      ok(me_attention_general_ext(q, kc, vc, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, out, t_, nh, nkv, d, dv, bs,
+                                  window, keep_first, v_table, v_pairing, scale, dtype_, items, stream_));
+      return;
+    }
     const bool mfma = dtype_ == kBF16 && me_attention_mfma_supported(d, bs) && group <= 16;
     const size_t mark = arena_.used;
     auto partials = [&](const SplitPlan& sp, float*& part_o, float*& part_ml) {
@@ -467,6 +510,19 @@ class Run {
                             scale, dtype_, items, stream_));
   }
 
+  // Linear attention with a decay per head over the state rows of the step's items.
+  void decay_state(const Op& op) {
+    const int heads = (int)op.i[0], d = (int)op.i[1], dv = (int)op.i[2], rd = (int)op.i[3];
+    const float* rope = (const float*)op.p[1];
+    if (rope && op.i[8] < s_.max_ctx)
+      throw Error(kBadValue, "the rotary table covers " + std::to_string(op.i[8]) + " positions, the step may reach " +
+                                 std::to_string(s_.max_ctx));
+    void* ws = arena_.take((size_t)me_decay_state_workspace(t_, heads, d, dv));
+    ok(me_decay_state(bufs_[op.in], rope, rd, (int)op.i[4], idx(s_.lay.positions), (const float*)op.p[0], (const float*)op.p[2],
+                      (float*)op.p[3], idx(s_.lay.item_start), idx(s_.lay.state_slots), bufs_[op.out], ws, t_, s_.lay.items, heads,
+                      d, dv, (int)op.i[5], op.f[0], (int)op.i[6], (int)op.i[7], op.f[1], dtype_, stream_));
+  }
+
   // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.
   void head(const Op& op) {
     const int rows = s_.lay.rows;
@@ -476,8 +532,13 @@ class Run {
       return;
     }
     void* picked = arena_.take((size_t)rows * h_ * elem_);
-    ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, (const float*)op.p[0], picked,
-                      idx(s_.lay.want_rows), rows, h_, op.f[0], 0, dtype_, stream_));
+    if (groups_of(op.i[0]) > 1 || pending_.scale != 1.f)
+      ok(me_add_group_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, pending_.scale,
+                              (const float*)op.p[0], picked, idx(s_.lay.want_rows), rows, h_, groups_of(op.i[0]), op.f[0], 0, dtype_,
+                              stream_));
+    else
+      ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, (const float*)op.p[0], picked,
+                        idx(s_.lay.want_rows), rows, h_, op.f[0], 0, dtype_, stream_));
     pending_ = Pending();
     logits_of(picked, op);
   }
@@ -558,7 +619,7 @@ std::vector<std::vector<int>> Program::prefill_geometries() const {
   std::vector<std::vector<int>> out;
   if (dtype_ != kBF16) return out;
   for (const Op& op : ops_) {
-    if (op.kind != kOpAttention) continue;
+    if (op.kind != kOpAttention || !attention_is_plain(op)) continue;
     const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], bs = (int)op.i[4], window = (int)op.i[5];
     if (!me_attention_mfma_supported(d, bs) || nh / nkv > 16) continue;
     std::vector<int> key = {nh, nkv, d, window};
@@ -578,7 +639,11 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
     if (op.kind == kOpNormLinear || op.kind == kOpLinear) need = (size_t)tokens * op.i[0] * 4 + pad;
     if (op.kind == kOpLinearDelta)  // up to 16 partial sums of up to 64 rows, or one float32 result of all rows
       need = std::max<size_t>((size_t)kMaxRuns * std::min<int64_t>(tokens, kSmallMaxRows), (size_t)tokens) * op.i[0] * 4 + pad;
-    if (op.kind == kOpAttention) {
+    if (op.kind == kOpDecayState)
+      need = (size_t)me_decay_state_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2]) + pad;
+    if (op.kind == kOpAttention && !attention_is_plain(op)) {
+      need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
+    } else if (op.kind == kOpAttention) {
       const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2];
       const int chunks = (nh / nkv + 15) / 16;
       size_t most = 0;  // items x splits at its largest over the batch sizes a launch may hold

@@ -24,22 +24,33 @@ namespace me {
 
 enum OpKind {
   kOpEmbed = 0,       // p0 table, f0 the multiplier on the looked-up rows; -> x
-  kOpNormLinear = 1,  // p0 norm weight, f0 eps, p1 W [rows, K], i0 rows of W, i1 K, i2 gated; pending + x -> out
-  kOpNorm = 2,        // p0 norm weight, f0 eps; pending + x -> out [tokens, hidden]
+  kOpNormLinear = 1,  // p0 norm weight, f0 eps, p1 W [rows, K], i0 rows of W, i1 K, i2 gated, i3 groups of the norm (0: one);
+                      // pending + x -> out
+  kOpNorm = 2,        // p0 norm weight, f0 eps, i0 groups of the norm (0: one); pending + x -> out [tokens, hidden]
   kOpLinear = 3,      // in, p1 W, i0 rows of W, i1 K, i2 gated -> out
-  kOpLinearDelta = 4, // in, p1 W, i0 rows of W (= hidden), i1 K -> pending
-  kOpDelta = 5,       // in -> pending
+  kOpLinearDelta = 4, // in, p1 W, i0 rows of W (= hidden), i1 K, f0 what the block multiplies the delta by (0: 1) -> pending
+  kOpDelta = 5,       // in, f0 what the block multiplies the delta by (0: 1) -> pending
   kOpAttention = 6,   // in qkv, p0 q-norm weight, p1 k-norm weight, p2 rotary table, p3 key pages, p4 value pages;
                       // i0 heads, i1 kv heads, i2 head size, i3 rotary size, i4 page size, i5 window, i6 writes pages,
-                      // i7 cache group, i8 positions the table covers; f0 eps, f1 scale -> out [tokens, heads * head size]
-  kOpHead = 7,        // p0 final norm weight, f0 eps, p1 head W [vocab, hidden], f1 the scale on the logits -> logits of the
-                      // wanted rows
+                      // i7 cache group, i8 positions the table covers; f0 eps, f1 scale -> out [tokens, heads * value size].
+                      // Beyond the plain form: i9 size of the value heads (0: the head size), i10 first keys that stay visible
+                      // behind the window, i11 pairing of the rotation (0: j with j + r/2; 1: 2j with 2j + 1), i12 values are
+                      // turned by their position and outputs turned back (0: no; 1 + the pairing), p5 the table of those angles
+  kOpHead = 7,        // p0 final norm weight, f0 eps, p1 head W [vocab, hidden], f1 the scale on the logits, i0 groups of the
+                      // norm (0: one) -> logits of the wanted rows
   kOpSample = 8,      // logits -> one token per wanted row
   kOpAdd = 9,         // pending + x -> x, as a kernel of its own (before a norm that is no RMS norm)
   kOpCall = 10,       // a part that brings its own code: p0 a function `int (const CallFrame*)`, p1 its context;
                       // in (or -1), out (or -1): the values it reads and writes. It launches on the step's stream.
   kOpHeadRows = 11,   // in: a value whose first rows are the normed wanted rows; p1 head W, f1 the scale on the logits
+  kOpDecayState = 12, // in: projections [tokens, heads (d | d | dv | dv)] (q, k, v, gate); p0 decay float32 [2, heads],
+                      // p1 rotary table, p2 weight of the norm over all heads, p3 the state rows [slots, heads, d, dv];
+                      // i0 heads, i1 d, i2 dv, i3 rotary size, i4 pairing, i5 activation of q, k, v, i6 kind of the output norm,
+                      // i7 activation of the gate, i8 positions the table covers; f0 scale on k, f1 eps
+                      // -> out [tokens, heads * dv]
 };
+
+constexpr int kOpInts = 16, kOpFloats = 4;
 
 // What a called part is handed (kOpCall). Pointers are device memory of this step: they change from step to step.
 struct CallFrame {
@@ -57,8 +68,8 @@ typedef int (*CallFn)(const CallFrame*);
 struct Op {
   int kind = 0, in = -1, out = -1;
   const void* p[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
-  int64_t i[10] = {0};
-  float f[2] = {0.f, 0.f};
+  int64_t i[kOpInts] = {0};
+  float f[kOpFloats] = {0.f, 0.f, 0.f, 0.f};
 };
 
 struct Value {

@@ -121,8 +121,8 @@ int me_runner_value(void* runner, int64_t cols, int elem) {
 int me_runner_op(void* runner, int kind, int in, int out, const void* const* ptrs, const int64_t* ints, const float* floats) {
   ME_RUN_GUARD(me::Op op; op.kind = kind; op.in = in; op.out = out;
                for (int i = 0; i < 6; ++i) op.p[i] = ptrs[i];
-               for (int i = 0; i < 10; ++i) op.i[i] = ints[i];
-               op.f[0] = floats[0]; op.f[1] = floats[1];
+               for (int i = 0; i < me::kOpInts; ++i) op.i[i] = ints[i];
+               for (int i = 0; i < me::kOpFloats; ++i) op.f[i] = floats[i];
                Runner* r = (Runner*)runner; r->prog.add_op(op); r->geometries = r->prog.prefill_geometries();
                return (int)r->prog.ops().size();)
 }

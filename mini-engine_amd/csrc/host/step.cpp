@@ -102,8 +102,9 @@ void Core::check_step(int vocab_size, bool scan_pages) const {
       if (!scan_pages) continue;
       const int w = config_.groups[g].window;
       const int first_key = w > 0 ? std::max(0, it.start - w + 1) : 0;
-      for (int i = first_key / bs; i < need; ++i)
-        if ((*table)[i] < 0)
+      const int kept_pages = w > 0 ? std::min(need, blocks_for(config_.groups[g].keep_first)) : 0;  // the kept first keys'
+      for (int i = 0; i < need; ++i)
+        if ((i < kept_pages || i >= first_key / bs) && (*table)[i] < 0)
           throw Error(kBadValue, "group " + std::to_string(g) + ": a page the step reads or writes was already given back");
     }
   }
@@ -242,8 +243,9 @@ void Core::refill(int32_t* dst, const StepLayout& lay, std::vector<RowMemo>& row
         have = 0;
       }
       const int first_key = window > 0 ? std::max(0, it->start - window + 1) : 0;
-      for (int p = std::max(have, first_key / bs); p < need; ++p)
-        if (table[p] < 0)
+      const int kept_pages = window > 0 ? std::min(need, blocks_for(config_.groups[g].keep_first)) : 0;
+      for (int p = have; p < need; ++p)
+        if ((p < kept_pages || p >= first_key / bs) && table[p] < 0)
           throw Error(kBadValue, "group " + std::to_string(g) + ": a page the step reads or writes was already given back");
       if (have < (int)table.size()) {
         std::copy(table.begin() + have, table.end(), out + have);

@@ -27,6 +27,25 @@ int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const float* k_w,
 int me_attention_general(const void* q, const void* k_cache, const void* v_cache, const int* positions,
                          const int* token_item, const int* block_table, int table_width, void* out, int num_tokens, int nh,
                          int nkv, int d, int bs, int window, float scale, int dtype, int items, hipStream_t stream);
+int me_attention_general_ext(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                             const int* token_item, const int* block_table, int table_width, void* out, int num_tokens, int nh,
+                             int nkv, int d, int dv, int bs, int window, int keep_first, const float* unturn, int un_pairing,
+                             float scale, int dtype, int items, hipStream_t stream);
+int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd, int pairing,
+                          const float* v_table, int v_pairing, const int* positions, const int* token_item,
+                          const int* block_table, int table_width, void* q_out, void* k_cache, void* v_cache, int num_tokens,
+                          int nh, int nkv, int d, int dv, int bs, float eps, int dtype, hipStream_t stream);
+int me_add_group_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, float delta_scale,
+                         const float* w, void* h, const int* rows, int num_rows, int dim, int groups, float eps, int write_x,
+                         int dtype, hipStream_t stream);
+int me_residual_add_scaled(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, float scale,
+                           int num_rows, int dim, int dtype, hipStream_t stream);
+int me_decay_state_padded_dim(int d);
+long long me_decay_state_workspace(long long tokens, int heads, int d, int dv);
+int me_decay_state(const void* proj, const float* rope_table, int rd, int pairing, const int* positions, const float* decay,
+                   const float* norm_w, float* state, const int* item_start, const int* state_slots, void* out, void* workspace,
+                   int num_tokens, int items, int heads, int d, int dv, int in_act, float key_scale, int norm_kind, int gate_act,
+                   float eps, int dtype, hipStream_t stream);
 int me_attention_mfma_supported(int d, int bs);
 int me_attention_decode_fused_supported(int d, int bs, int rotary_dim, int group);
 int me_attention_prefill_columns(int wide);

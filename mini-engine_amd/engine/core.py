@@ -117,7 +117,8 @@ def _layout_dict(out: np.ndarray, groups: int) -> dict:
 
 
 class HostCore:
-    """Owner of the native core object. ``groups`` is a list of ``(window, num_pages)``."""
+    """Owner of the native core object. ``groups`` is a list of ``(window, num_pages)`` or
+    ``(window, num_pages, keep_first)``: with a window, the first ``keep_first`` keys of a request stay."""
 
     def __init__(self, block_size: int, groups: list[tuple[int, int]], enable_prefix_caching: bool = True,
                  num_state_slots: int = 0, has_state: bool = False, max_num_seqs: int = 1 << 20,
@@ -126,7 +127,7 @@ class HostCore:
         self.block_size, self.num_groups = int(block_size), len(groups)
         settings = _ints([block_size, int(bool(enable_prefix_caching)), num_state_slots, int(bool(has_state)), max_num_seqs,
                           max_num_batched_tokens, max_model_len])
-        flat = _ints([v for g in groups for v in g])
+        flat = _ints([v for g in groups for v in (g[0], g[1], g[2] if len(g) > 2 else 0)])
         eos = _ints(sorted(int(e) for e in eos_token_ids))
         self._box = self._L.me_core_new(_ptr(settings), _ptr(flat), len(groups), _ptr(eos), len(eos),
                                         ctypes.c_uint64(seed & ((1 << 64) - 1)))

@@ -28,7 +28,8 @@ from ..ops.library import lib
 _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 _declared = False
 
-EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS = range(12)
+EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS, DECAY_STATE = range(13)
+OP_INTS, OP_FLOATS = 16, 4  # csrc/host/program.h: kOpInts, kOpFloats
 _RAISES = {1: ValueError, 2: RuntimeError, 3: AssertionError}
 
 
@@ -102,8 +103,8 @@ class Normed:
     product where the step is small enough); ``value()`` gives the normed activations as a value of
     their own."""
 
-    def __init__(self, program: "StepProgram", weight: torch.Tensor, eps: float):
-        self.program, self.weight, self.eps = program, weight, float(eps)
+    def __init__(self, program: "StepProgram", weight: torch.Tensor, eps: float, groups: int = 1):
+        self.program, self.weight, self.eps, self.groups = program, weight, float(eps), int(groups)
         self.used = False
         self._value: int | None = None
 
@@ -111,7 +112,7 @@ class Normed:
         if self._value is None:
             p = self.program
             self._value = p.take(p.hidden, p.elem)
-            p.op(NORM, out=self._value, ptrs=[self.weight], floats=[self.eps])
+            p.op(NORM, out=self._value, ptrs=[self.weight], ints=[self.groups], floats=[self.eps])
             p.pending_consumed()
             self.used = True
         return self._value
@@ -150,6 +151,7 @@ class StepProgram:
         self._scopes: list[list[int]] = []
         self._pending_value: int | None = None
         self.num_ops = 0
+        self.delta_scale = 1.0  # what the block being written multiplies its parts' results by (set by the block)
         self.draws = False
         self.last_prefill_columns = 0  # query columns of the prefill attention's blocks in the last eager step (0: none ran)
         # called parts: their C trampolines (kept alive), the memory and the batch of the step that is running,
@@ -208,8 +210,8 @@ class StepProgram:
                     raise ValueError("a step program holds contiguous tensors only")
                 self._keep.append(t)
                 p[i] = t.data_ptr()
-        iv = (ctypes.c_int64 * 10)(*[int(v) for v in ints])
-        fv = (ctypes.c_float * 2)(*[float(v) for v in floats])
+        iv = (ctypes.c_int64 * OP_INTS)(*[int(v) for v in ints])
+        fv = (ctypes.c_float * OP_FLOATS)(*[float(v) for v in floats])
         self.num_ops = _ok(self._L.me_runner_op(self.handle, kind, in_, out, p, iv, fv))
 
     def embed(self, table: torch.Tensor, multiplier: float = 1.0) -> None:
@@ -222,7 +224,7 @@ class StepProgram:
         float32 weight and its eps)."""
         weight, eps = norm.as_fused()
         self._want(weight, torch.float32, (self.hidden,), "norm weight")
-        return Normed(self, weight, eps)
+        return Normed(self, weight, eps, getattr(norm, "groups", 1))
 
     def linear(self, x, weight: torch.Tensor, gated: "bool | str" = False) -> int:
         """``x @ weight.T`` (``gated``, True or the name of an activation: ``act(gate) * up`` with the weight's
@@ -239,7 +241,7 @@ class StepProgram:
         if isinstance(x, Normed) and x._value is None:
             if k != self.hidden:
                 raise ValueError("a product behind the norm reads the hidden size")
-            self.op(NORM_LINEAR, out=out, ptrs=[x.weight, weight], ints=[rows, k, gate], floats=[x.eps])
+            self.op(NORM_LINEAR, out=out, ptrs=[x.weight, weight], ints=[rows, k, gate, x.groups], floats=[x.eps])
             x.used = True
             self.pending_consumed()
             return out
@@ -254,23 +256,31 @@ class StepProgram:
         rows, k = weight.shape
         self._want(weight, self.dtype, (self.hidden, self._value_kinds[x][0]), "weight")
         out = self.take(rows)
-        self.op(LINEAR_DELTA, in_=x, out=out, ptrs=[None, weight], ints=[rows, k])
+        self.op(LINEAR_DELTA, in_=x, out=out, ptrs=[None, weight], ints=[rows, k], floats=[self.delta_scale])
         self._pending_value = out
 
     def delta(self, x: int) -> None:
         """A value ``[tokens, hidden]`` in the compute dtype as the part's result."""
         if self._value_kinds[x] != (self.hidden, self.elem):
             raise ValueError("a part's result has the hidden size and the compute dtype")
-        self.op(DELTA, in_=x)
+        self.op(DELTA, in_=x, floats=[self.delta_scale])
         self._pending_value = x
 
     def attention(self, qkv: int, *, q_norm: torch.Tensor | None, k_norm: torch.Tensor | None, rope: torch.Tensor | None,
                   k_cache: torch.Tensor, v_cache: torch.Tensor, heads: int, kv_heads: int, head_dim: int, block_size: int,
-                  window: int, writes: bool, group: int, eps: float, scale: float) -> int:
+                  window: int, writes: bool, group: int, eps: float, scale: float, value_dim: int | None = None,
+                  keep_first: int = 0, pairing: int = 0, value_rope: torch.Tensor | None = None, value_pairing: int = 0) -> int:
         """Per-head q/k norm, rotation, page write and causal attention over the request's pages for a
         value ``[tokens, (heads + 2 kv_heads) head_dim]`` (``writes`` false: ``[tokens, heads head_dim]``,
-        the pages are another layer's); returns the value ``[tokens, heads head_dim]``."""
-        cols = (heads + (2 * kv_heads if writes else 0)) * head_dim
+        the pages are another layer's); returns the value ``[tokens, heads head_dim]``.
+
+        ``value_dim``: the value heads' size where it is not ``head_dim`` (the input then ends in ``kv_heads``
+        heads of that size and the result has ``heads * value_dim`` columns); ``keep_first``: the first keys that stay
+        visible behind the window; ``pairing``: 0 pairs element j with j + r/2, 1 pairs 2j with 2j + 1;
+        ``value_rope`` / ``value_pairing``: the table ``[positions, 2, value_dim / 2]`` that the values are turned by
+        before they are cached and the outputs turned back by."""
+        dv = head_dim if value_dim is None else int(value_dim)
+        cols = heads * head_dim + (kv_heads * (head_dim + dv) if writes else 0)
         if self._value_kinds[qkv] != (cols, self.elem):
             raise ValueError(f"the attention's input has {self._value_kinds[qkv][0]} columns, not {cols}")
         rotary_dim = covers = 0
@@ -279,10 +289,42 @@ class StepProgram:
             rotary_dim, covers = 2 * rope.shape[2], rope.shape[0]
             if covers < self.max_positions:
                 raise ValueError(f"the rotary table covers {covers} positions of {self.max_positions}")
-        out = self.take(heads * head_dim)
-        self.op(ATTENTION, in_=qkv, out=out, ptrs=[q_norm, k_norm, rope, k_cache, v_cache],
-                ints=[heads, kv_heads, head_dim, rotary_dim, block_size, window, int(writes), group, covers],
+        turned = 0
+        if value_rope is not None:
+            self._want(value_rope, torch.float32, None, "table of the values' angles")
+            if 2 * value_rope.shape[2] != dv or value_rope.shape[0] < self.max_positions:
+                raise ValueError(f"the values' table must cover {self.max_positions} positions and {dv} elements")
+            turned = 1 + int(value_pairing)
+        out = self.take(heads * dv)
+        self.op(ATTENTION, in_=qkv, out=out, ptrs=[q_norm, k_norm, rope, k_cache, v_cache, value_rope],
+                ints=[heads, kv_heads, head_dim, rotary_dim, block_size, window, int(writes), group, covers,
+                      0 if dv == head_dim else dv, keep_first, pairing, turned],
                 floats=[eps, scale])
+        return out
+
+    def decay_state(self, proj: int, *, decay: torch.Tensor, rope: torch.Tensor | None, pairing: int, norm_weight: torch.Tensor | None,
+                    state: torch.Tensor, heads: int, key_dim: int, value_dim: int, input_act: int, key_scale: float,
+                    norm_kind: int, gate_act: int, eps: float) -> int:
+        """Linear attention with a decay per head over the step's items, from and into their rows of ``state``
+        ``[slots, heads, key_dim, value_dim]`` (float32), for a value ``[tokens, heads (2 key_dim + 2 value_dim)]`` (q, k,
+        v and gate projections); returns the value ``[tokens, heads * value_dim]`` that the output projection reads."""
+        cols = 2 * heads * (key_dim + value_dim)
+        if self._value_kinds[proj] != (cols, self.elem):
+            raise ValueError(f"the projections have {self._value_kinds[proj][0]} columns, not {cols}")
+        self._want(decay, torch.float32, (2, heads), "decay")
+        self._want(state, torch.float32, (state.shape[0], heads, key_dim, value_dim), "state")
+        if norm_weight is not None:
+            self._want(norm_weight, torch.float32, (heads * value_dim,), "weight of the output norm")
+        rotary_dim = covers = 0
+        if rope is not None:
+            self._want(rope, torch.float32, None, "rotary table")
+            rotary_dim, covers = 2 * rope.shape[2], rope.shape[0]
+            if covers < self.max_positions:
+                raise ValueError(f"the rotary table covers {covers} positions of {self.max_positions}")
+        out = self.take(heads * value_dim)
+        self.op(DECAY_STATE, in_=proj, out=out, ptrs=[decay, rope, norm_weight, state],
+                ints=[heads, key_dim, value_dim, rotary_dim, pairing, input_act, norm_kind, gate_act, covers],
+                floats=[key_scale, eps])
         return out
 
     def add(self) -> None:
@@ -311,7 +353,7 @@ class StepProgram:
         self._calls.append(c_fn)
         p = (ctypes.c_void_p * 6)()
         p[0] = ctypes.cast(c_fn, ctypes.c_void_p).value
-        iv, fv = (ctypes.c_int64 * 10)(), (ctypes.c_float * 2)()
+        iv, fv = (ctypes.c_int64 * OP_INTS)(), (ctypes.c_float * OP_FLOATS)()
         self.num_ops = _ok(self._L.me_runner_op(self.handle, CALL, in_, out, p, iv, fv))
         return out
 
@@ -345,7 +387,7 @@ class StepProgram:
         """Final norm of the wanted rows, the head product, the logits times ``logit_scale``."""
         norm_weight, eps = norm.as_fused()
         self._want(weight, self.dtype, (self.vocab, self.hidden), "head")
-        self.op(HEAD, ptrs=[norm_weight, weight], floats=[eps, logit_scale])
+        self.op(HEAD, ptrs=[norm_weight, weight], ints=[getattr(norm, "groups", 1)], floats=[eps, logit_scale])
         self.pending_consumed()
 
     def sample(self) -> None:

@@ -75,7 +75,7 @@ class ModelRunner:
                                     self.num_state_slots, self.dtype, self.device)
         self.num_groups = len(self.layout.groups)
         self.max_blocks_per_seq = -(-config.max_model_len // config.block_size)
-        self.core = HostCore(config.block_size, [(g.window, g.num_blocks or config.num_blocks) for g in self.layout.groups],
+        self.core = HostCore(config.block_size, [(g.window, g.num_blocks or config.num_blocks, g.keep_first) for g in self.layout.groups],
                              config.enable_prefix_caching, self.num_state_slots, self.layout.has_state, config.max_num_seqs,
                              config.max_num_batched_tokens, config.max_model_len, eos_token_ids, config.seed)
         self.program = StepProgram(self.dtype, decoder.plan.hidden_size, decoder.plan.vocab_size, config.max_model_len)

@@ -154,6 +154,63 @@ def add_rmsnorm(
     return out
 
 
+def add_group_rmsnorm(
+    x: torch.Tensor,
+    delta: "torch.Tensor | PartialSums | None",
+    weight: torch.Tensor,
+    eps: float,
+    dtype: torch.dtype,
+    groups: int = 1,
+    delta_scale: float = 1.0,
+    out: torch.Tensor | None = None,
+    rows: torch.Tensor | None = None,
+    write_x: bool = True,
+) -> torch.Tensor:
+    """As :func:`add_rmsnorm` with ``x += delta_scale * delta`` and the norm taken over ``groups`` equal consecutive
+    parts of a row, each divided by its own root mean square."""
+    _want(x, "x", torch.float32, (None, None))
+    t, d = x.shape
+    _want(weight, "weight", torch.float32, (d,))
+    if groups < 1 or d % groups:
+        raise ValueError(f"a row of {d} elements cannot be cut into {groups} equal groups")
+    parts = None
+    if isinstance(delta, PartialSums):
+        parts, delta = delta.parts, None
+        _want(parts, "partial sums", torch.float32, (None, t, d))
+    elif delta is not None:
+        _want(delta, "delta", dtype, (t, d))
+    n = t
+    if rows is not None:
+        _want(rows, "rows", torch.int32)
+        n = rows.numel()
+    if out is None:
+        out = torch.empty((n, d), dtype=dtype, device=x.device)
+    _want(out, "out", dtype, (n, d))
+    check(lib().me_add_group_rmsnorm(_p(x), _p(delta), _p(parts), _i(0 if parts is None else parts.shape[0]),
+                                     ctypes.c_longlong(0 if parts is None else t * d), _f(delta_scale), _p(weight), _p(out),
+                                     _p(rows), _i(n), _i(d), _i(groups), _f(eps), _i(1 if write_x else 0), _i(_code(dtype)),
+                                     _stream()))
+    return out
+
+
+def residual_add_scaled(x: torch.Tensor, delta: "torch.Tensor | PartialSums", scale: float) -> torch.Tensor:
+    """``x += scale * delta`` in place for the float32 residual stream [T, D] and a delta in float32 or bfloat16 (or
+    partial sums)."""
+    _want(x, "x", torch.float32, (None, None))
+    t, d = x.shape
+    parts, code = None, _F32
+    if isinstance(delta, PartialSums):
+        parts, delta = delta.parts, None
+        _want(parts, "partial sums", torch.float32, (None, t, d))
+    else:
+        _want(delta, "delta", None, (t, d))
+        code = _code(delta.dtype)
+    check(lib().me_residual_add_scaled(_p(x), _p(delta), _p(parts), _i(0 if parts is None else parts.shape[0]),
+                                       ctypes.c_longlong(0 if parts is None else t * d), _f(scale), _i(t), _i(d), _i(code),
+                                       _stream()))
+    return x
+
+
 def residual_add(x: torch.Tensor, delta: "torch.Tensor | PartialSums") -> torch.Tensor:
     """``x += delta`` in place for the float32 residual stream [T, D] and a delta in the compute dtype
     (or partial sums): the add alone, for a norm that runs as a part of its own."""
@@ -217,9 +274,75 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor | None = None, activation: s
 # ------------------------------------------------------------------------------------- attention
 
 
-def _check_cache(k_cache, v_cache, dtype, nkv, d, bs):
+def _check_cache(k_cache, v_cache, dtype, nkv, d, bs, dv=None):
     _want(k_cache, "k_cache", dtype, (None, nkv, bs, d))
-    _want(v_cache, "v_cache", dtype, (k_cache.shape[0], nkv, d, bs))
+    _want(v_cache, "v_cache", dtype, (k_cache.shape[0], nkv, d if dv is None else dv, bs))
+
+
+def qkv_rotate_scatter(qkv, q_w, k_w, rope, pairing, v_table, v_pairing, positions, token_item, block_table, k_cache, v_cache,
+                       nh: int, nkv: int, d: int, dv: int, eps: float, q_out: torch.Tensor | None = None) -> torch.Tensor:
+    """Per-head q/k norm (``q_w`` / ``k_w`` float32 [d] or None), rotation of the first elements of q and k by the angles
+    of ``rope`` [P, 2, r/2] (``pairing`` 0: j with j + r/2; 1: 2j with 2j + 1), values turned over all ``dv`` elements by
+    ``v_table`` [P, 2, dv/2] (or copied), keys and values written to their pages. ``qkv`` is ``[T, nh d + nkv d + nkv dv]``;
+    returns q ``[T, nh, d]``. Every position must lie inside the tables and in a page of the token's table row."""
+    _want(qkv, "qkv", None, (None, nh * d + nkv * (d + dv)))
+    t = qkv.shape[0]
+    bs = k_cache.shape[2]
+    _check_cache(k_cache, v_cache, qkv.dtype, nkv, d, bs, dv)
+    _check_step_index(positions, token_item, block_table, t)
+    rd = 0
+    for w, name in ((q_w, "q_w"), (k_w, "k_w")):
+        if w is not None:
+            _want(w, name, torch.float32, (d,))
+    if rope is not None:
+        _want(rope, "rope", torch.float32, (None, 2, None))
+        rd = 2 * rope.shape[2]
+    if v_table is not None:
+        _want(v_table, "v_table", torch.float32, (None, 2, dv // 2))
+    if q_out is None:
+        q_out = torch.empty((t, nh, d), dtype=qkv.dtype, device=qkv.device)
+    _want(q_out, "q_out", qkv.dtype, (t, nh, d))
+    check(lib().me_qkv_rotate_scatter(_p(qkv), _p(q_w), _p(k_w), _p(rope), _i(rd), _i(pairing), _p(v_table), _i(v_pairing),
+                                      _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]), _p(q_out),
+                                      _p(k_cache), _p(v_cache), _i(t), _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _f(eps),
+                                      _i(_code(qkv.dtype)), _stream()))
+    return q_out
+
+
+def decay_state(proj, rope, pairing, positions, decay, norm_w, state, item_start, state_slots, heads: int, d: int, dv: int,
+                in_act: int, key_scale: float, norm_kind: int, gate_act: int, eps: float,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    """Linear attention with a decay per head (``csrc/decay_state.hip``) over the items of a step. ``proj``
+    ``[T, 2 heads (d + dv)]`` holds the q, k, v and gate projections; ``decay`` float32 [2, heads]; ``state`` float32
+    ``[slots, heads, d, dv]`` is read and written at the rows ``state_slots`` [items]; ``item_start`` [items + 1] cuts the
+    tokens into items. Returns ``[T, heads * dv]`` in the dtype of ``proj``."""
+    _want(proj, "proj", None, (None, 2 * heads * (d + dv)))
+    t = proj.shape[0]
+    _want(positions, "positions", torch.int32, (t,))
+    _want(decay, "decay", torch.float32, (2, heads))
+    _want(state, "state", torch.float32, (None, heads, d, dv))
+    _want(item_start, "item_start", torch.int32)
+    _want(state_slots, "state_slots", torch.int32)
+    items = state_slots.numel()
+    if item_start.numel() != items + 1:
+        raise ValueError("item_start has one entry more than there are items")
+    rd = 0
+    if rope is not None:
+        _want(rope, "rope", torch.float32, (None, 2, None))
+        rd = 2 * rope.shape[2]
+    if norm_w is not None:
+        _want(norm_w, "norm_w", torch.float32, (heads * dv,))
+    if out is None:
+        out = torch.empty((t, heads * dv), dtype=proj.dtype, device=proj.device)
+    _want(out, "out", proj.dtype, (t, heads * dv))
+    L = lib()
+    L.me_decay_state_workspace.restype = ctypes.c_longlong
+    need = L.me_decay_state_workspace(ctypes.c_longlong(t), _i(heads), _i(d), _i(dv))
+    ws = torch.empty(need, dtype=torch.uint8, device=proj.device)
+    check(L.me_decay_state(_p(proj), _p(rope), _i(rd), _i(pairing), _p(positions), _p(decay), _p(norm_w), _p(state),
+                           _p(item_start), _p(state_slots), _p(out), _p(ws), _i(t), _i(items), _i(heads), _i(d), _i(dv),
+                           _i(in_act), _f(key_scale), _i(norm_kind), _i(gate_act), _f(eps), _i(_code(proj.dtype)), _stream()))
+    return out
 
 
 def _check_step_index(positions, token_item, block_table, t):
@@ -309,22 +432,29 @@ def attention_general(
     window: int = 0,
     out: torch.Tensor | None = None,
     shared_tiles: bool = True,
+    keep_first: int = 0,
+    unturn: torch.Tensor | None = None,
+    un_pairing: int = 0,
 ) -> torch.Tensor:
-    """Causal grouped-query attention of q [T, nh, d] over the paged cache; returns [T, nh * d]. float32 steps with
-    two and more tokens per row of the block table go to a kernel whose blocks share the tiles of keys and values among
-    their tokens (``shared_tiles=False``: the kernel with a wave per token and head for every step; the same bits)."""
+    """Causal grouped-query attention of q [T, nh, d] over the paged cache; returns [T, nh * dv] (dv: the size of the
+    cached value heads). float32 steps with two and more tokens per row of the block table go to a kernel whose blocks
+    share the tiles of keys and values among their tokens (``shared_tiles=False``: the kernel with a wave per token and
+    head for every step; the same bits). ``keep_first``: the first keys that stay visible behind the window;
+    ``unturn`` float32 [P, 2, dv/2]: the angles every output row is turned back by (``un_pairing`` as for the rotation)."""
     _want(q, "q", None, (None, None, None))
     t, nh, d = q.shape
-    nkv, bs = k_cache.shape[1], k_cache.shape[2]
-    _check_cache(k_cache, v_cache, q.dtype, nkv, d, bs)
+    nkv, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
+    _check_cache(k_cache, v_cache, q.dtype, nkv, d, bs, dv)
     _check_step_index(positions, token_item, block_table, t)
+    if unturn is not None:
+        _want(unturn, "unturn", torch.float32, (None, 2, dv // 2))
     if out is None:
-        out = torch.empty((t, nh * d), dtype=q.dtype, device=q.device)
-    _want(out, "out", q.dtype, (t, nh * d))
-    check(lib().me_attention_general(
+        out = torch.empty((t, nh * dv), dtype=q.dtype, device=q.device)
+    _want(out, "out", q.dtype, (t, nh * dv))
+    check(lib().me_attention_general_ext(
         _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]),
-        _p(out), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(_code(q.dtype)),
-        _i(block_table.shape[0] if shared_tiles else 0), _stream()))
+        _p(out), _i(t), _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _i(window), _i(keep_first), _p(unturn), _i(un_pairing),
+        _f(scale), _i(_code(q.dtype)), _i(block_table.shape[0] if shared_tiles else 0), _stream()))
     return out
 
 

@@ -1,6 +1,6 @@
 """Parts of a decoder layer. Importing this package registers the built-in kinds."""
 
-from . import attention, mlp, norm, rotary  # noqa: F401
+from . import attention, decay_state, mlp, norm, rotary  # noqa: F401
 from .base import (
     BLOCK_ARRANGEMENTS,
     FEED_FORWARDS,
@@ -16,7 +16,7 @@ from .base import (
     StateBinding,
     StateNeed,
 )
-from .block import PreNormBlock, build_block
+from .block import ParallelBlock, PreNormBlock, build_block
 from .decoder import Decoder
 
 __all__ = [
@@ -31,6 +31,7 @@ __all__ = [
     "NORMS",
     "Norm",
     "POSITION_ENCODINGS",
+    "ParallelBlock",
     "PositionEncoding",
     "PreNormBlock",
     "StateBinding",

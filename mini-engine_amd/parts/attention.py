@@ -9,6 +9,12 @@ window), then the output projection.
 Sizes and constants all come from the spec: head counts, head size, score scale, eps of the q/k
 norm (None: no norm), window (0: none), position encoding (None: none), and ``cache_from`` (read
 another layer's pages and write none).
+
+Beyond that plain form the spec may give the value heads a size of their own, keep the first keys of a
+request visible behind the window, pair neighbouring elements in the rotation, and have the values turned
+by their position before they are cached (every output is then turned back by its query's position). A
+layer that uses any of these runs the kernels that take every size (``qkv_rotate_scatter``,
+``attention_general``), in both dtypes.
 """
 
 from __future__ import annotations
@@ -32,49 +38,73 @@ class Attention(Mixer):
             raise ValueError(f"the score scale must be positive and finite, got {s.scale}: the kernels scale before they mask")
         if s.num_heads % s.num_kv_heads:
             raise ValueError(f"{s.num_heads} query heads are not a multiple of {s.num_kv_heads} key/value heads")
-        if s.head_dim % 16 or not 16 <= s.head_dim <= MAX_HEAD_DIM:
-            raise ValueError(f"head_dim={s.head_dim} is not supported: the attention kernels take head sizes "
-                             f"from 16 to {MAX_HEAD_DIM} in steps of 16")
         if s.window < 0:
             raise ValueError(f"window={s.window} must be >= 0")
         self.nh, self.nkv, self.d = s.num_heads, s.num_kv_heads, s.head_dim
+        self.dv = int(getattr(s, "v_dim", s.head_dim))
+        self.keep_first = int(getattr(s, "keep_first", 0))
+        if self.keep_first < 0 or (self.keep_first and not s.window):
+            raise ValueError(f"keep_first={self.keep_first} must be >= 0 and needs a window")
         self.position = None if s.position is None else POSITION_ENCODINGS.build(s.position, dtype, device)
+        vp = getattr(s, "value_position", None)
+        self.value_position = None if vp is None else POSITION_ENCODINGS.build(vp, dtype, device)
+        if self.value_position is not None and self.value_position.rotary_dim != self.dv:
+            raise ValueError(f"values of size {self.dv} are turned over all of their elements, not {self.value_position.rotary_dim}")
+        self.pairing = 0 if self.position is None else int(getattr(self.position, "pairing_code", 0))
+        # the plain form: what the matrix-core kernels and the fused decode prologue are written for
+        self.plain = self.dv == self.d and not self.keep_first and self.pairing == 0 and self.value_position is None
+        if self.plain and (s.head_dim % 16 or not 16 <= s.head_dim <= MAX_HEAD_DIM):
+            raise ValueError(f"head_dim={s.head_dim} is not supported: the attention kernels take head sizes "
+                             f"from 16 to {MAX_HEAD_DIM} in steps of 16")
+        if not self.plain:
+            if not (1 <= self.d <= MAX_HEAD_DIM and 1 <= self.dv <= MAX_HEAD_DIM):
+                raise ValueError(f"head sizes {self.d} and {self.dv} must be in 1..{MAX_HEAD_DIM}")
+            if s.cache_from is not None:
+                raise ValueError("an attention layer beyond the plain form owns its pages")
+        names = dict(getattr(s, "names", ()) or ())
+        self._n = {r: names.get(r, d) for r, d in (("q", "q_proj.weight"), ("k", "k_proj.weight"), ("v", "v_proj.weight"),
+                                                    ("o", "o_proj.weight"), ("q_norm", "q_norm.weight"),
+                                                    ("k_norm", "k_norm.weight"))}
         self.q_norm_w = self.k_norm_w = None
         self.w_qkv = self.w_o = None
 
     # ---- weights
     def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
         s = self.spec
+        n = self._n
         wants = {
-            f"{prefix}.q_proj.weight": TensorWant((s.num_heads * s.head_dim, s.hidden_size)),
-            f"{prefix}.o_proj.weight": TensorWant((s.hidden_size, s.num_heads * s.head_dim)),
+            f"{prefix}.{n['q']}": TensorWant((s.num_heads * s.head_dim, s.hidden_size)),
+            f"{prefix}.{n['o']}": TensorWant((s.hidden_size, s.num_heads * self.dv)),
         }
         if s.cache_from is None:
-            wants[f"{prefix}.k_proj.weight"] = TensorWant((s.num_kv_heads * s.head_dim, s.hidden_size))
-            wants[f"{prefix}.v_proj.weight"] = TensorWant((s.num_kv_heads * s.head_dim, s.hidden_size))
+            wants[f"{prefix}.{n['k']}"] = TensorWant((s.num_kv_heads * s.head_dim, s.hidden_size))
+            wants[f"{prefix}.{n['v']}"] = TensorWant((s.num_kv_heads * self.dv, s.hidden_size))
         if s.qk_norm_eps is not None:
-            wants[f"{prefix}.q_norm.weight"] = TensorWant((s.head_dim,), "vector")
+            wants[f"{prefix}.{n['q_norm']}"] = TensorWant((s.head_dim,), "vector")
             if s.cache_from is None:
-                wants[f"{prefix}.k_norm.weight"] = TensorWant((s.head_dim,), "vector")
+                wants[f"{prefix}.{n['k_norm']}"] = TensorWant((s.head_dim,), "vector")
         return wants
 
     def load(self, tensors, prefix: str) -> None:
         s = self.spec
-        q = tensors[f"{prefix}.q_proj.weight"]
+        n = self._n
+        q = tensors[f"{prefix}.{n['q']}"]
         if s.cache_from is None:
-            self.w_qkv = torch.cat((q, tensors[f"{prefix}.k_proj.weight"], tensors[f"{prefix}.v_proj.weight"]), dim=0)
+            self.w_qkv = torch.cat((q, tensors[f"{prefix}.{n['k']}"], tensors[f"{prefix}.{n['v']}"]), dim=0)
         else:
             self.w_qkv = q.contiguous()
-        self.w_o = tensors[f"{prefix}.o_proj.weight"]
+        self.w_o = tensors[f"{prefix}.{n['o']}"]
         if s.qk_norm_eps is not None:
-            self.q_norm_w = tensors[f"{prefix}.q_norm.weight"]
-            self.k_norm_w = tensors.get(f"{prefix}.k_norm.weight")
+            self.q_norm_w = tensors[f"{prefix}.{n['q_norm']}"]
+            self.k_norm_w = tensors.get(f"{prefix}.{n['k_norm']}")
 
     # ---- cache
     def cache_need(self):
         if self.spec.cache_from is not None:
             return None
-        return KVCacheNeed(self.nkv, self.d, self.spec.window)
+        if self.plain:
+            return KVCacheNeed(self.nkv, self.d, self.spec.window)
+        return KVCacheNeed(self.nkv, self.d, self.spec.window, value_dim=self.dv, keep_first=self.keep_first)
 
     def cache_source(self):
         return self.spec.cache_from
@@ -91,6 +121,14 @@ class Attention(Mixer):
         table = batch.block_table(b.group)
         rope = None if self.position is None else self.position.tables(batch.max_ctx)
         eps = 0.0 if s.qk_norm_eps is None else float(s.qk_norm_eps)
+        if not self.plain:
+            vt = None if self.value_position is None else self.value_position.tables(batch.max_ctx)
+            v_pairing = 0 if self.value_position is None else self.value_position.pairing_code
+            q = K.qkv_rotate_scatter(proj, self.q_norm_w, self.k_norm_w, rope, self.pairing, vt, v_pairing, batch.positions,
+                                     batch.token_item, table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, self.dv, eps)
+            out = K.attention_general(q, b.k_cache, b.v_cache, batch.positions, batch.token_item, table, float(s.scale),
+                                      int(s.window), keep_first=self.keep_first, unturn=vt, un_pairing=v_pairing)
+            return K.linear(out, self.w_o, as_delta=True)
         if (self.dtype is torch.bfloat16 and batch.decode_only and K.attention_decode_fused_supported(
                 self.d, b.block_size, 0 if rope is None else 2 * rope.shape[2], self.nh // self.nkv)):
             # one new token per item: norm, rotary, page write and attention in one launch
@@ -117,7 +155,10 @@ class Attention(Mixer):
             rope=None if self.position is None else self.position.tables(program.max_positions),
             k_cache=b.k_cache, v_cache=b.v_cache, heads=self.nh, kv_heads=self.nkv, head_dim=self.d,
             block_size=b.block_size, window=int(s.window), writes=owns, group=b.group,
-            eps=0.0 if s.qk_norm_eps is None else float(s.qk_norm_eps), scale=float(s.scale))
+            eps=0.0 if s.qk_norm_eps is None else float(s.qk_norm_eps), scale=float(s.scale),
+            value_dim=self.dv, keep_first=self.keep_first, pairing=self.pairing,
+            value_rope=None if self.value_position is None else self.value_position.tables(program.max_positions),
+            value_pairing=0 if self.value_position is None else self.value_position.pairing_code)
         program.linear_delta(out, self.w_o)
 
     def attend(self, q: torch.Tensor, batch, table: torch.Tensor, b: KVBinding) -> torch.Tensor:

@@ -50,6 +50,12 @@ class KVCacheNeed:
     num_kv_heads: int
     head_dim: int
     window: int = 0  # 0: every earlier key stays needed
+    value_dim: int | None = None  # size of the value heads (None: head_dim)
+    keep_first: int = 0  # with a window: the first keys of a request stay needed as well
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)

@@ -4,6 +4,12 @@
 
     x = x + mixer(norm1(x));  x = x + ffn(norm2(x))
 
+``parallel``::
+
+    h = norm1(x);  x = x + scale * (mixer(h) + ffn(h))
+
+one norm that both parts read; ``scale`` is the layer spec's ``residual_scale``; the feed-forward may be absent.
+
 The residual stream ``x`` is kept in float32 and every sum into it is a float32 sum. A block returns
 its feed-forward output unadded; the next norm kernel (of the next block, or the model's final norm)
 adds it while it norms, so each residual add costs no pass of its own.
@@ -57,7 +63,58 @@ class PreNormBlock:
                     program.delta(out)
 
 
+class ParallelBlock:
+    """One norm; the mixer and the feed-forward both read its output; their sum, times the spec's ``residual_scale``,
+    is added to the stream. The mixer's result is added by a kernel of its own (the feed-forward does not wait for it:
+    it reads the normed activations); the feed-forward's stays pending for the next norm, like a pre-norm block's."""
+
+    def __init__(self, spec, dtype: torch.dtype, device: torch.device):
+        self.spec, self.dtype = spec, dtype
+        self.mixer = MIXERS.build(spec.mixer, dtype, device)
+        self.ffn = None if spec.ffn is None else FEED_FORWARDS.build(spec.ffn, dtype, device)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, dtype, device)
+        self.ffn_norm = None
+        self.scale = float(spec.residual_scale)
+
+    def weight_wants(self):
+        s = self.spec
+        wants = {}
+        wants.update(self.mixer_norm.weight_wants(s.mixer_norm_name))
+        wants.update(self.mixer.weight_wants(s.mixer_prefix))
+        if self.ffn is not None:
+            wants.update(self.ffn.weight_wants(s.ffn_prefix))
+        return wants
+
+    def load(self, tensors) -> None:
+        s = self.spec
+        self.mixer_norm.load(tensors, s.mixer_norm_name)
+        self.mixer.load(tensors, s.mixer_prefix)
+        if self.ffn is not None:
+            self.ffn.load(tensors, s.ffn_prefix)
+
+    def emit(self, program, cache=None) -> None:
+        parts = [(self.mixer, (cache,))] + ([(self.ffn, ())] if self.ffn is not None else [])
+        norm = self.mixer_norm
+        with program.scope():
+            h = program.normed(norm) if norm.as_fused() is not None else program.normed_by(norm)
+            h.value()  # the normed activations as a value of their own: two parts read them
+            before, program.delta_scale = program.delta_scale, self.scale
+            try:
+                for at, (part, extra) in enumerate(parts):
+                    if callable(getattr(part, "emit", None)):
+                        out = part.emit(program, h, *extra)
+                    else:
+                        out = program.call_part(part, h, extra)
+                    if out is not None:
+                        program.delta(out)
+                    if at + 1 < len(parts):
+                        program.add()  # the last part's result waits for the next norm instead
+            finally:
+                program.delta_scale = before
+
+
 BLOCK_ARRANGEMENTS.register("pre_norm", PreNormBlock)
+BLOCK_ARRANGEMENTS.register("parallel", ParallelBlock)
 
 
 def build_block(spec, dtype, device):

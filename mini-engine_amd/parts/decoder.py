@@ -74,6 +74,8 @@ class Decoder:
         for i in set(self.plan.order):
             parts += [self.blocks[i].mixer, self.blocks[i].ffn, self.blocks[i].mixer_norm, self.blocks[i].ffn_norm]
         for obj in parts:
+            if obj is None:  # a block without a feed-forward, or with one norm for both parts
+                continue
             for v in vars(obj).values():
                 if isinstance(v, torch.Tensor):
                     add(v)
@@ -101,4 +103,4 @@ class Decoder:
         for i in set(self.plan.order):
             b = self.blocks[i]
             parts += [b.mixer, b.ffn, b.mixer_norm, b.ffn_norm]
-        return all(getattr(p, "graph_safe", False) for p in parts)
+        return all(getattr(p, "graph_safe", False) for p in parts if p is not None)

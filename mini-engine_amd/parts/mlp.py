@@ -20,18 +20,21 @@ class GatedMlp(FeedForward):
         if spec.activation not in K.GATE_ACTIVATIONS:
             raise ValueError(f"gated_mlp knows the activations {sorted(K.GATE_ACTIVATIONS)}, got {spec.activation!r}")
         self.w_gate_up = self.w_down = None
+        names = dict(getattr(spec, "names", ()) or ())
+        self._gate, self._up, self._down = (names.get(r, d) for r, d in (("gate", "gate_proj.weight"), ("up", "up_proj.weight"),
+                                                                         ("down", "down_proj.weight")))
 
     def weight_wants(self, prefix: str) -> dict[str, TensorWant]:
         s = self.spec
         return {
-            f"{prefix}.gate_proj.weight": TensorWant((s.intermediate_size, s.hidden_size)),
-            f"{prefix}.up_proj.weight": TensorWant((s.intermediate_size, s.hidden_size)),
-            f"{prefix}.down_proj.weight": TensorWant((s.hidden_size, s.intermediate_size)),
+            f"{prefix}.{self._gate}": TensorWant((s.intermediate_size, s.hidden_size)),
+            f"{prefix}.{self._up}": TensorWant((s.intermediate_size, s.hidden_size)),
+            f"{prefix}.{self._down}": TensorWant((s.hidden_size, s.intermediate_size)),
         }
 
     def load(self, tensors, prefix: str) -> None:
-        self.w_gate_up = torch.cat((tensors[f"{prefix}.gate_proj.weight"], tensors[f"{prefix}.up_proj.weight"]), dim=0)
-        self.w_down = tensors[f"{prefix}.down_proj.weight"]
+        self.w_gate_up = torch.cat((tensors[f"{prefix}.{self._gate}"], tensors[f"{prefix}.{self._up}"]), dim=0)
+        self.w_down = tensors[f"{prefix}.{self._down}"]
 
     takes_normed_input = True
 

@@ -1,5 +1,6 @@
 """RMSNorm part: ``x * rsqrt(mean(x^2) + eps) * weight`` in float32
-(reference: ``src/mini_engine/model.py:59-69``; the weight multiplies directly, eps inside the root)."""
+(reference: ``src/mini_engine/model.py:59-69``; the weight multiplies directly, eps inside the root). With
+``groups > 1`` the row is cut into that many equal consecutive parts and each is divided by its own root mean square."""
 
 from __future__ import annotations
 
@@ -17,6 +18,9 @@ class RMSNorm(Norm):
         super().__init__(spec, dtype, device)
         self.eps = float(spec.eps)
         self.dim = int(spec.dim)
+        self.groups = int(getattr(spec, "groups", 1))
+        if self.groups < 1 or self.dim % self.groups:
+            raise ValueError(f"a norm over {self.dim} elements cannot be cut into {self.groups} equal groups")
         self.weight = torch.ones(self.dim, dtype=torch.float32, device=device)
 
     def weight_wants(self, name: str) -> dict[str, TensorWant]:
@@ -29,6 +33,8 @@ class RMSNorm(Norm):
         return self.weight, self.eps
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.groups > 1:
+            return K.add_group_rmsnorm(x, None, self.weight, self.eps, self.dtype, groups=self.groups, write_x=False)
         return K.add_rmsnorm(x, None, self.weight, self.eps, self.dtype, write_x=False)
 
     def __call__(self, x: torch.Tensor) -> torch.Tensor:
