@@ -117,7 +117,7 @@ def main(argv: list[str] | None = None) -> int:
                     help="most tokens live requests hold at any time (each rounded up to 64); sizes the cache pool")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--num-blocks", type=int, default=None, help="pages of the cache pool (instead of --max-tokens)")
-    ap.add_argument("--max-live", type=int, default=8,
+    ap.add_argument("--max-live", type=int, default=4,
                     help="largest batch a decode graph is captured for; state slots of models with per-request state")
     args = ap.parse_args(argv)
     if args.max_tokens is None and args.num_blocks is None:
