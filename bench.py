@@ -114,7 +114,8 @@ class DecodeBench:
     """An engine of one shape and dtype at a fixed context length, for decode steps at several batch
     sizes and whole-prompt prefills."""
 
-    def __init__(self, cfg, dtype: str, ctx: int, max_batch: int, budget: int = 8192, block: int = 16, seed: int = 0):
+    def __init__(self, cfg, dtype: str, ctx: int, max_batch: int, budget: int = 8192, block: int = 16, seed: int = 0,
+                 architecture: str = "Qwen3ForCausalLM"):
         import torch
 
         from mini_engine_amd import EngineConfig, LLMEngine
@@ -124,7 +125,8 @@ class DecodeBench:
         self.econf = EngineConfig(block_size=block, num_blocks=max_batch * blocks_per_seq + 256, max_num_seqs=max_batch,
                                   max_num_batched_tokens=budget, max_model_len=ctx, enable_prefix_caching=False,
                                   dtype=dtype, seed=0, cuda_graphs=True)
-        self.engine = LLMEngine.from_random("Qwen3ForCausalLM", cfg, self.econf, seed=seed)
+        self.engine = LLMEngine.from_random(architecture, cfg, self.econf, seed=seed)
+        self.vocab = self.engine.model.plan.vocab_size
         self.gen = torch.Generator().manual_seed(0)
         self.kv_per_token = self.engine.runner.storage.kv_bytes_per_token()
         self.weight_bytes = self.engine.model.weight_bytes()
@@ -132,7 +134,7 @@ class DecodeBench:
     def prompt(self, n: int) -> list[int]:
         import torch
 
-        return torch.randint(100, self.cfg.vocab_size, (n,), generator=self.gen).tolist()
+        return torch.randint(100, self.vocab, (n,), generator=self.gen).tolist()
 
     def prefill(self, tokens: int) -> dict:
         """One whole prompt through the step function: best of three after a warm-up."""
@@ -154,6 +156,8 @@ class DecodeBench:
 
         once()
         s = min(once() for _ in range(3))
+        if not hasattr(self.cfg, "num_attention_heads"):  # another design: its caller prices the prompt
+            return {"value": round(tokens / s, 1), "tokens": tokens, "ms": round(s * 1e3, 3)}
         return {"value": round(tokens / s, 1), "tokens": tokens, "ms": round(s * 1e3, 3),
                 "frac": round(prefill_flops(self.cfg, tokens) / s / PEAK_FLOPS[self.dtype], 4)}
 
@@ -339,6 +343,67 @@ def shape_line(shape: str, args) -> dict:
     }
 
 
+# Layer sizes that resemble a real model's, for the Gonurax design beside the Qwen3 dense design at equal sizes: width,
+# feed-forward, heads of 128 (keys and values), 8 key/value heads in the attention layers; eight layers, of which the
+# Gonurax model has two attention layers (a window of 1,024 keys that keeps the first 4), two lightning and four
+# retention layers; a vocabulary of 32,768.
+DESIGN_SIZES = {"1024": dict(width=1024, ff=3072, heads=16), "2048": dict(width=2048, ff=6144, heads=16)}
+DESIGN_LAYERS, DESIGN_VOCAB = 8, 32768
+
+
+def gonurax_config(size: str):
+    from mini_engine_amd.models.gonurax import GonuraxConfig
+
+    z = DESIGN_SIZES[size]
+    h = z["heads"]
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": h, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "mask": {"size": 1024, "keep_first": 4},
+                     "rot": {"base": 1e6, "dims": 128}}}
+    decay = [1.0 - 2.0 ** -(5 + 7 * i / max(1, h - 1)) for i in range(h)]
+    lit = {"type": "lightning", "mlp": mlp, "mixer": {"heads": h, "dim": 128, "vdim": 128, "decay": decay}}
+    ret = {"type": "retention", "mlp": mlp, "mixer": {"heads": h, "dim": 128, "vdim": 128, "decay": decay, "rot": {"base": 1e6, "dims": 128}}}
+    order = [att, lit, ret, ret] * (DESIGN_LAYERS // 4)
+    return GonuraxConfig.from_dict({"architecture": "Gonurax", "vocab": DESIGN_VOCAB, "width": z["width"], "residual_mult": 0.7,
+                                    "norm": {"eps": 1e-6, "groups": 2}, "layers": order})
+
+
+def design_line(args) -> dict:
+    """Prefill and decode throughput of the Gonurax design beside the Qwen3 dense design at equal layer sizes (random
+    weights, eight layers): a 2,048-token prompt, and decode steps at batch 1, 8 and 64 behind a context of 2,304."""
+    from mini_engine_amd.models.qwen3 import Qwen3Config
+
+    ctx, out = 2304, {}
+    sizes = [z for z in args.design_sizes.split(",") if z]
+    for size in sizes:
+        z = DESIGN_SIZES[size]
+        qwen = Qwen3Config(vocab_size=DESIGN_VOCAB, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, num_hidden_layers=DESIGN_LAYERS,
+                           hidden_size=z["width"], num_attention_heads=z["heads"], num_key_value_heads=8,
+                           intermediate_size=z["ff"], tie_word_embeddings=True, max_position_embeddings=40960)
+        for name, arch, cfg in (("gonurax", "Gonurax", gonurax_config(size)), ("qwen3", "Qwen3ForCausalLM", qwen)):
+            bench = DecodeBench(cfg, args.dtype, ctx, 64, architecture=arch)
+            pf = bench.prefill(args.prefill_tokens)
+            out[f"{name}_{size}_prefill_{pf['tokens']}_tok_s"] = pf["value"]
+            out[f"{name}_{size}_prefill_{pf['tokens']}_ms"] = pf["ms"]
+            for b in (1, 8, 64):
+                m = bench.decode(b, args.steps, args.warmup)
+                out[f"{name}_{size}_decode_b{b}_tok_s"] = round(m[0], 1)
+                out[f"{name}_{size}_decode_b{b}_ms_per_step"] = round(m[1], 4)
+            bench.engine = None
+            del bench
+            release()
+    first = sizes[0]
+    return {"metric": f"decode tok/s at batch 8 (Gonurax design, width {DESIGN_SIZES[first]['width']}, {DESIGN_LAYERS} layers)",
+            "value": out[f"gonurax_{first}_decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": out[f"gonurax_{first}_decode_b8_ms_per_step"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights",
+            "config": {"model": "Gonurax design beside the Qwen3 dense design at equal layer sizes", "layers": DESIGN_LAYERS,
+                       "vocab": DESIGN_VOCAB, "sizes": {z: DESIGN_SIZES[z] for z in sizes}, "seq_len": ctx, "global_batch": 8,
+                       "parallelism": "single GPU"},
+            "points": out}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -353,10 +418,16 @@ def main() -> int:
     ap.add_argument("--skip-prefill", action="store_true", help="profiling aid: do not measure the prefill")
     ap.add_argument("--skip-extras", action="store_true",
                     help="profiling aid: only the decode steps and the prefill (no serving workloads, no float32 point, no probes)")
+    ap.add_argument("--design", default="", choices=["", "gonurax"],
+                    help="instead of the default workload: this design beside the Qwen3 dense design at equal layer sizes")
+    ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design to measure, comma separated")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")
         return 2
+    if args.design:
+        print(json.dumps(design_line(args)))
+        return 0
     if args.shape != "0.6b":
         print(json.dumps(shape_line(args.shape, args)))
         return 0
