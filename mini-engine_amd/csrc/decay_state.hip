@@ -4,7 +4,7 @@
 //   S_t = decay_h * S_(t-1) + k_t v_t^T        (S: [d, dv], float32, kept in a slot between steps)
 //   o_t = S_t^T q_t
 //
-// Three kernels a step. `decay_state_prepare` turns the projections [T, H*d | H*d | H*dv | ...] into float32 q, k
+// Three kernels a step (five where long prompts are walked a chunk at a time). `decay_state_prepare` turns the projections [T, H*d | H*d | H*dv | ...] into float32 q, k
 // and v: an optional activation, an optional rotation of the first rd elements of q and k by the position's angles
 // (either pairing), and a scale on k. `decay_state_scan` walks the new tokens of every item in order, from the state
 // in the item's slot, and leaves the new state there. `decay_state_finish` norms the outputs (every head by its own
@@ -78,69 +78,150 @@ __global__ __launch_bounds__(256) void decay_state_prepare_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------- scan
-// Grid (item, head, 64 columns); a wave owns 16 columns of the state: lane = rg * 16 + column, rg = 0..3 the quarter of
-// the rows (RPL rows a lane, 4 * RPL >= d; q32 and k32 rows are padded to 4 * RPL with zeros). The next token's q, k
-// and v are requested before the current token's arithmetic.
-template <int RPL>
+// A wave owns 16 columns of the state: lane = rg * 16 + column, rg = 0..3 the quarter of the rows (RPL rows a lane,
+// 4 * RPL >= d; q32 and k32 rows are padded to 4 * RPL with zeros). The next token's q, k and v are requested before
+// the current token's arithmetic. Three forms:
+//
+//   DS_WHOLE   grid (item, head, 64 columns): the item's new tokens in order, from the state in its slot, which is left
+//              updated. The decay is applied as two floats. Decode steps and short portions.
+//   DS_SUMS    grid (chunk of 64 tokens, head, 64 columns): the chunk's own sum  U = sum_s decay^(last - s) k_s v_s^T,
+//              from nothing, into the chunk's place of `chunks` [chunk, head, d, dv]; no outputs.
+//   DS_OUTPUTS the same grid: the chunk's tokens in order from the state at the chunk's start, which
+//              `decay_state_chunk_starts_kernel` has put in the chunk's place; outputs, no state written.
+//
+// With the last two a long prompt is walked by all its chunks at once: sums, then the states at the chunks' starts (a
+// pass over the chunks per element, with decay^64 worked out in double), then outputs. Inside a chunk the decay is one
+// float: over 64 tokens what the float misses of the configured value stays below 1e-5 of a term.
+#define DS_CHUNK 64
+enum DsMode { DS_WHOLE = 0, DS_SUMS = 1, DS_OUTPUTS = 2 };
+
+// The item and the tokens of chunk `c` (counted over all items of the step, ceil(tokens / 64) chunks an item).
+__device__ __forceinline__ bool ds_chunk_tokens(const int* __restrict__ item_start, int items, int c, int& item, int& t0, int& t1) {
+  int base = 0;
+  for (int i = 0; i < items; ++i) {
+    const int a = item_start[i], n = item_start[i + 1] - a;
+    const int nc = (n + DS_CHUNK - 1) / DS_CHUNK;
+    if (c < base + nc) {
+      item = i;
+      t0 = a + (c - base) * DS_CHUNK;
+      t1 = min(t0 + DS_CHUNK, a + n);
+      return true;
+    }
+    base += nc;
+  }
+  return false;
+}
+
+template <int RPL, int MODE>
 __global__ __launch_bounds__(256) void decay_state_scan_kernel(
     const float* __restrict__ q32, const float* __restrict__ k32, const float* __restrict__ v32, float* __restrict__ o32,
-    float* __restrict__ state, const float* __restrict__ decay, const int* __restrict__ item_start,
-    const int* __restrict__ state_slots, int heads, int d, int dv) {
+    float* __restrict__ state, float* __restrict__ chunks, const float* __restrict__ decay, const int* __restrict__ item_start,
+    const int* __restrict__ state_slots, int items, int heads, int d, int dv) {
   constexpr int DP = 4 * RPL;
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
-  const int item = blockIdx.x, head = blockIdx.y;
+  const int head = blockIdx.y;
   const int col = (blockIdx.z * 4 + wave) * 16 + (lane & 15), rg = lane >> 4;
   if ((blockIdx.z * 4 + wave) * 16 >= dv) return;  // (whole waves: no block-wide barrier below)
   const bool has_col = col < dv;
-  const int t0 = item_start[item], t1 = item_start[item + 1];
+  int item = blockIdx.x, t0, t1;
+  if (MODE == DS_WHOLE) {
+    t0 = item_start[item], t1 = item_start[item + 1];
+  } else if (!ds_chunk_tokens(item_start, items, blockIdx.x, item, t0, t1)) {
+    return;
+  }
   const int slot = state_slots[item];
   if (slot < 0 || t1 <= t0) return;
-  const float lam = decay[head], lam_lo = decay[heads + head];
-  float* srow = state + (((size_t)slot * heads + head) * d) * dv;  // [d, dv]
+  const float lam = decay[head], lam_lo = MODE == DS_WHOLE ? decay[heads + head] : 0.f;
+  float* srow = MODE == DS_WHOLE ? state + (((size_t)slot * heads + head) * d) * dv
+                                 : chunks + (((size_t)blockIdx.x * heads + head) * d) * dv;  // [d, dv]
   float S[RPL];
 #pragma unroll
   for (int r = 0; r < RPL; ++r) {
     const int i = rg * RPL + r;
-    S[r] = has_col && i < d ? srow[(size_t)i * dv + col] : 0.f;
+    S[r] = MODE != DS_SUMS && has_col && i < d ? srow[(size_t)i * dv + col] : 0.f;
   }
   float4 qn[RPL / 4], kn[RPL / 4];
   float vn;
   auto fetch = [&](int t) {
-    const float4* qp = reinterpret_cast<const float4*>(q32 + ((size_t)t * heads + head) * DP + rg * RPL);
     const float4* kp = reinterpret_cast<const float4*>(k32 + ((size_t)t * heads + head) * DP + rg * RPL);
 #pragma unroll
-    for (int r = 0; r < RPL / 4; ++r) qn[r] = qp[r], kn[r] = kp[r];
+    for (int r = 0; r < RPL / 4; ++r) kn[r] = kp[r];
+    if (MODE != DS_SUMS) {
+      const float4* qp = reinterpret_cast<const float4*>(q32 + ((size_t)t * heads + head) * DP + rg * RPL);
+#pragma unroll
+      for (int r = 0; r < RPL / 4; ++r) qn[r] = qp[r];
+    }
     vn = has_col ? v32[((size_t)t * heads + head) * dv + col] : 0.f;
   };
   fetch(t0);
   for (int t = t0; t < t1; ++t) {
     float4 qc[RPL / 4], kc[RPL / 4];
 #pragma unroll
-    for (int r = 0; r < RPL / 4; ++r) qc[r] = qn[r], kc[r] = kn[r];
+    for (int r = 0; r < RPL / 4; ++r) kc[r] = kn[r];
+    if (MODE != DS_SUMS) {
+#pragma unroll
+      for (int r = 0; r < RPL / 4; ++r) qc[r] = qn[r];
+    }
     const float vc = vn;
     if (t + 1 < t1) fetch(t + 1);
     float o = 0.f;
 #pragma unroll
     for (int r = 0; r < RPL / 4; ++r) {
       const float kk[4] = {kc[r].x, kc[r].y, kc[r].z, kc[r].w};
-      const float qq[4] = {qc[r].x, qc[r].y, qc[r].z, qc[r].w};
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const float s = S[4 * r + u];
-        const float sn = fmaf(lam_lo, s, fmaf(lam, s, kk[u] * vc));
+        float sn = fmaf(lam, s, kk[u] * vc);
+        if (MODE == DS_WHOLE) sn = fmaf(lam_lo, s, sn);
         S[4 * r + u] = sn;
-        o = fmaf(sn, qq[u], o);
+      }
+      if (MODE != DS_SUMS) {
+        const float qq[4] = {qc[r].x, qc[r].y, qc[r].z, qc[r].w};
+#pragma unroll
+        for (int u = 0; u < 4; ++u) o = fmaf(S[4 * r + u], qq[u], o);
       }
     }
-    o += __shfl_xor(o, 16, ME_WAVE);
-    o += __shfl_xor(o, 32, ME_WAVE);
-    if (rg == 0 && has_col) o32[((size_t)t * heads + head) * dv + col] = o;
+    if (MODE != DS_SUMS) {
+      o += __shfl_xor(o, 16, ME_WAVE);
+      o += __shfl_xor(o, 32, ME_WAVE);
+      if (rg == 0 && has_col) o32[((size_t)t * heads + head) * dv + col] = o;
+    }
   }
+  if (MODE == DS_OUTPUTS) return;
 #pragma unroll
   for (int r = 0; r < RPL; ++r) {
     const int i = rg * RPL + r;
     if (has_col && i < d) srow[(size_t)i * dv + col] = S[r];
   }
+}
+
+// The states at the chunks' starts, in place of the chunks' sums: per item, head and element of the state,
+// S = state[slot]; for each chunk of the item in order: (sum, place) = (place, S); S = decay^(chunk's tokens) * S + sum;
+// state[slot] = S. Grid (elements / 256, head, item).
+__global__ __launch_bounds__(256) void decay_state_chunk_starts_kernel(float* __restrict__ state, float* __restrict__ chunks,
+                                                                        const float* __restrict__ decay,
+                                                                        const int* __restrict__ item_start,
+                                                                        const int* __restrict__ state_slots, int heads,
+                                                                        int elements) {
+  const int e = blockIdx.x * 256 + threadIdx.x, head = blockIdx.y, item = blockIdx.z;
+  if (e >= elements) return;
+  const int slot = state_slots[item];
+  const int n = item_start[item + 1] - item_start[item];
+  if (slot < 0 || n <= 0) return;
+  int base = 0;
+  for (int i = 0; i < item; ++i) base += (item_start[i + 1] - item_start[i] + DS_CHUNK - 1) / DS_CHUNK;
+  const double lam = (double)decay[head] + (double)decay[heads + head];
+  const int nc = (n + DS_CHUNK - 1) / DS_CHUNK, tail = n - (nc - 1) * DS_CHUNK;
+  const float full = (float)pow(lam, (double)DS_CHUNK), last = (float)pow(lam, (double)tail);
+  float* sp = state + ((size_t)slot * heads + head) * elements + e;
+  float S = *sp;
+  for (int c = 0; c < nc; ++c) {
+    float* place = chunks + ((size_t)(base + c) * heads + head) * elements + e;
+    const float sum = *place;
+    *place = S;
+    S = fmaf(c + 1 < nc ? full : last, S, sum);
+  }
+  *sp = S;
 }
 
 // ----------------------------------------------------------------------------------------------- finish
@@ -186,10 +267,12 @@ extern "C" int me_decay_state_padded_dim(int d) {  // the row length of the prep
   return d <= 32 ? 32 : d <= 64 ? 64 : d <= 128 ? 128 : 256;
 }
 
-// Bytes of float32 workspace that a step of `tokens` tokens needs (prepared q, k, v and the raw outputs).
-extern "C" long long me_decay_state_workspace(long long tokens, int heads, int d, int dv) {
+// Bytes of float32 workspace that a step of `tokens` tokens in `items` items needs: prepared q, k, v, the raw outputs,
+// and a state per chunk of 64 tokens (at most tokens / 64 + items of them) for steps that walk their chunks side by side.
+extern "C" long long me_decay_state_workspace(long long tokens, long long items, int heads, int d, int dv) {
   const long long dp = me_decay_state_padded_dim(d);
-  return tokens * heads * (2 * dp + 2 * (long long)dv) * 4 + 1024;
+  const long long chunks = tokens / DS_CHUNK + items;
+  return tokens * heads * (2 * dp + 2 * (long long)dv) * 4 + chunks * heads * (long long)d * dv * 4 + 1024;
 }
 
 // proj [T, proj_cols]: q heads, k heads (d each), v heads, gate (dv each), so proj_cols = 2 heads (d + dv).
@@ -199,7 +282,7 @@ extern "C" int me_decay_state(const void* proj, const float* rope_table, int rd,
                               const float* decay, const float* norm_w, float* state, const int* item_start,
                               const int* state_slots, void* out, void* workspace, int num_tokens, int items, int heads, int d,
                               int dv, int in_act, float key_scale, int norm_kind, int gate_act, float eps, int dtype,
-                              hipStream_t stream) {
+                              int longest_item, hipStream_t stream) {
   if (num_tokens <= 0 || items <= 0) return 0;
   if (heads <= 0 || heads > DS_MAX_D || d <= 0 || d > DS_MAX_D || dv <= 0)
     return me_fail("me_decay_state: heads=%d d=%d dv=%d (heads and key size up to %d)", heads, d, dv, DS_MAX_D);
@@ -207,7 +290,7 @@ extern "C" int me_decay_state(const void* proj, const float* rope_table, int rd,
     return me_fail("me_decay_state: rotary_dim=%d with head size %d, pairing %d", rd, d, pairing);
   if (norm_kind != 0 && norm_kind != 1) return me_fail("me_decay_state: norm kind %d", norm_kind);
   if (norm_kind == 1 && !norm_w) return me_fail("me_decay_state: the norm over all heads needs its weight");
-  if (items > 65535 * 16 || heads > 65535) return me_fail("me_decay_state: %d items, %d heads", items, heads);
+  if (items > 65535 || heads > 65535) return me_fail("me_decay_state: %d items, %d heads", items, heads);
   if ((uintptr_t)workspace & 15) return me_fail("me_decay_state: the workspace must be aligned to 16 bytes");
   const int dp = me_decay_state_padded_dim(d);
   const int proj_cols = 2 * heads * (d + dv);
@@ -217,11 +300,28 @@ extern "C" int me_decay_state(const void* proj, const float* rope_table, int rd,
   float* o32 = v32 + (size_t)num_tokens * heads * dv;
   const long long units = (long long)num_tokens * heads * 3;
   const unsigned prep_blocks = (unsigned)((units + 3) / 4);
-  const dim3 scan_grid(items, heads, (dv + 63) / 64);
-  if (scan_grid.z > 65535) return me_fail("me_decay_state: value heads of %d elements", dv);
-#define DS_SCAN(RPL)                                                                                                        \
-  decay_state_scan_kernel<RPL><<<scan_grid, 256, 0, stream>>>(q32, k32, v32, o32, state, decay, item_start, state_slots, heads, \
-                                                              d, dv)
+  float* chunk_states = o32 + (size_t)num_tokens * heads * dv;
+  // An item of more than two chunks (`longest_item`: the most tokens an item brings, 0 if unknown): all chunks of the
+  // step side by side. Else every item in order, a block per item, head and 64 columns.
+  const bool by_chunks = longest_item > 2 * DS_CHUNK;
+  const int num_chunks = num_tokens / DS_CHUNK + items;  // an upper bound: blocks beyond the last chunk leave at once
+  const dim3 scan_grid(by_chunks ? num_chunks : items, heads, (dv + 63) / 64);
+  if (scan_grid.z > 65535 || (long long)d * dv > (1ll << 24)) return me_fail("me_decay_state: value heads of %d elements", dv);
+  const dim3 starts_grid((d * dv + 255) / 256, heads, items);
+#define DS_SCAN_MODE(RPL, MODE)                                                                                              \
+  decay_state_scan_kernel<RPL, MODE><<<scan_grid, 256, 0, stream>>>(q32, k32, v32, o32, state, chunk_states, decay, item_start, \
+                                                                    state_slots, items, heads, d, dv)
+#define DS_SCAN(RPL)                                                                                                         \
+  do {                                                                                                                       \
+    if (by_chunks) {                                                                                                         \
+      DS_SCAN_MODE(RPL, DS_SUMS);                                                                                            \
+      decay_state_chunk_starts_kernel<<<starts_grid, 256, 0, stream>>>(state, chunk_states, decay, item_start, state_slots,     \
+                                                                       heads, d * dv);                                        \
+      DS_SCAN_MODE(RPL, DS_OUTPUTS);                                                                                         \
+    } else {                                                                                                                 \
+      DS_SCAN_MODE(RPL, DS_WHOLE);                                                                                           \
+    }                                                                                                                        \
+  } while (0)
 #define DS_RUN(T)                                                                                                           \
   do {                                                                                                                      \
     decay_state_prepare_kernel<T><<<prep_blocks, 256, 0, stream>>>((const T*)proj, proj_cols, rope_table, rd, pairing,        \
@@ -244,5 +344,6 @@ extern "C" int me_decay_state(const void* proj, const float* rope_table, int rd,
     DS_RUN(bf16_t);
 #undef DS_RUN
 #undef DS_SCAN
+#undef DS_SCAN_MODE
   return me_check_launch("me_decay_state");
 }

@@ -517,10 +517,13 @@ class Run {
     if (rope && op.i[8] < s_.max_ctx)
       throw Error(kBadValue, "the rotary table covers " + std::to_string(op.i[8]) + " positions, the step may reach " +
                                  std::to_string(s_.max_ctx));
-    void* ws = arena_.take((size_t)me_decay_state_workspace(t_, heads, d, dv));
+    void* ws = arena_.take((size_t)me_decay_state_workspace(t_, s_.lay.items, heads, d, dv));
+    int longest = 0;  // (a replayed decode step has no host-side lengths: every item brings one token)
+    if (!s_.decode_only && s_.qlens)
+      for (int i = 0; i < s_.lay.items; ++i) longest = std::max(longest, s_.qlens[i]);
     ok(me_decay_state(bufs_[op.in], rope, rd, (int)op.i[4], idx(s_.lay.positions), (const float*)op.p[0], (const float*)op.p[2],
                       (float*)op.p[3], idx(s_.lay.item_start), idx(s_.lay.state_slots), bufs_[op.out], ws, t_, s_.lay.items, heads,
-                      d, dv, (int)op.i[5], op.f[0], (int)op.i[6], (int)op.i[7], op.f[1], dtype_, stream_));
+                      d, dv, (int)op.i[5], op.f[0], (int)op.i[6], (int)op.i[7], op.f[1], dtype_, longest, stream_));
   }
 
   // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.
@@ -640,7 +643,7 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
     if (op.kind == kOpLinearDelta)  // up to 16 partial sums of up to 64 rows, or one float32 result of all rows
       need = std::max<size_t>((size_t)kMaxRuns * std::min<int64_t>(tokens, kSmallMaxRows), (size_t)tokens) * op.i[0] * 4 + pad;
     if (op.kind == kOpDecayState)
-      need = (size_t)me_decay_state_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2]) + pad;
+      need = (size_t)me_decay_state_workspace(tokens, items, (int)op.i[0], (int)op.i[1], (int)op.i[2]) + pad;
     if (op.kind == kOpAttention && !attention_is_plain(op)) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
     } else if (op.kind == kOpAttention) {

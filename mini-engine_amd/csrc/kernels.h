@@ -41,11 +41,11 @@ int me_add_group_rmsnorm(void* x, const void* delta, const float* parts, int num
 int me_residual_add_scaled(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, float scale,
                            int num_rows, int dim, int dtype, hipStream_t stream);
 int me_decay_state_padded_dim(int d);
-long long me_decay_state_workspace(long long tokens, int heads, int d, int dv);
+long long me_decay_state_workspace(long long tokens, long long items, int heads, int d, int dv);
 int me_decay_state(const void* proj, const float* rope_table, int rd, int pairing, const int* positions, const float* decay,
                    const float* norm_w, float* state, const int* item_start, const int* state_slots, void* out, void* workspace,
                    int num_tokens, int items, int heads, int d, int dv, int in_act, float key_scale, int norm_kind, int gate_act,
-                   float eps, int dtype, hipStream_t stream);
+                   float eps, int dtype, int longest_item, hipStream_t stream);
 int me_attention_mfma_supported(int d, int bs);
 int me_attention_decode_fused_supported(int d, int bs, int rotary_dim, int group);
 int me_attention_prefill_columns(int wide);

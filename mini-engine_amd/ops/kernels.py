@@ -311,11 +311,12 @@ def qkv_rotate_scatter(qkv, q_w, k_w, rope, pairing, v_table, v_pairing, positio
 
 def decay_state(proj, rope, pairing, positions, decay, norm_w, state, item_start, state_slots, heads: int, d: int, dv: int,
                 in_act: int, key_scale: float, norm_kind: int, gate_act: int, eps: float,
-                out: torch.Tensor | None = None) -> torch.Tensor:
+                out: torch.Tensor | None = None, longest_item: int = 0) -> torch.Tensor:
     """Linear attention with a decay per head (``csrc/decay_state.hip``) over the items of a step. ``proj``
     ``[T, 2 heads (d + dv)]`` holds the q, k, v and gate projections; ``decay`` float32 [2, heads]; ``state`` float32
     ``[slots, heads, d, dv]`` is read and written at the rows ``state_slots`` [items]; ``item_start`` [items + 1] cuts the
-    tokens into items. Returns ``[T, heads * dv]`` in the dtype of ``proj``."""
+    tokens into items. ``longest_item``: the most tokens an item brings (beyond 128 the step's chunks of 64 tokens are
+    walked side by side; 0: every item in order). Returns ``[T, heads * dv]`` in the dtype of ``proj``."""
     _want(proj, "proj", None, (None, 2 * heads * (d + dv)))
     t = proj.shape[0]
     _want(positions, "positions", torch.int32, (t,))
@@ -337,11 +338,12 @@ def decay_state(proj, rope, pairing, positions, decay, norm_w, state, item_start
     _want(out, "out", proj.dtype, (t, heads * dv))
     L = lib()
     L.me_decay_state_workspace.restype = ctypes.c_longlong
-    need = L.me_decay_state_workspace(ctypes.c_longlong(t), _i(heads), _i(d), _i(dv))
+    need = L.me_decay_state_workspace(ctypes.c_longlong(t), ctypes.c_longlong(items), _i(heads), _i(d), _i(dv))
     ws = torch.empty(need, dtype=torch.uint8, device=proj.device)
     check(L.me_decay_state(_p(proj), _p(rope), _i(rd), _i(pairing), _p(positions), _p(decay), _p(norm_w), _p(state),
                            _p(item_start), _p(state_slots), _p(out), _p(ws), _i(t), _i(items), _i(heads), _i(d), _i(dv),
-                           _i(in_act), _f(key_scale), _i(norm_kind), _i(gate_act), _f(eps), _i(_code(proj.dtype)), _stream()))
+                           _i(in_act), _f(key_scale), _i(norm_kind), _i(gate_act), _f(eps), _i(_code(proj.dtype)),
+                           _i(longest_item), _stream()))
     return out
 
 

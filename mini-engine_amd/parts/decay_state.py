@@ -99,7 +99,7 @@ class DecayState(Mixer):
         rope = None if self.position is None else self.position.tables(batch.max_ctx)
         out = K.decay_state(proj, rope, self.pairing, batch.positions, self.decay, self.norm_w, cache.state, batch.item_start,
                             batch.state_slots, self.h, self.d, self.dv, in_act, float(s.key_scale), norm_kind, gate_act,
-                            float(s.norm_eps))
+                            float(s.norm_eps), longest_item=0 if batch.decode_only else int(batch.max_qlen))
         return K.linear(out, self.w_o, as_delta=True)
 
     def emit(self, program, h, cache: StateBinding | None = None) -> None:

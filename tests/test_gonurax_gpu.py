@@ -191,8 +191,8 @@ def test_decay_state_kernels_in_portions_and_beside_other_items(heads, d, dv, rd
     slot = {"a": 4, "b": 1, "c": 2}
     fed = {r: 0 for r in lens}
     got = {r: [] for r in lens}
-    plan = [[("a", 300), ("b", 1), ("c", 2)], [("b", 30), ("a", 1), ("c", 100)], [("c", 47), ("a", 1)], [("a", 118), ("c", 1), ("b", 6)],
-            [("d", 33)]]
+    # (steps whose longest portion has more than two chunks of 64 tokens walk all chunks side by side: the first two)
+    plan = [[("a", 300), ("b", 1), ("c", 2)], [("b", 30), ("a", 1), ("c", 147)], [("a", 119), ("c", 1), ("b", 6)], [("d", 33)]]
     for step in plan:
         if step[0][0] == "d":
             slot["d"] = slot.pop("b")  # b is over: its slot is used again
@@ -207,7 +207,8 @@ def test_decay_state_kernels_in_portions_and_beside_other_items(heads, d, dv, rd
         out = K.decay_state(torch.cat(rows).cuda().contiguous(), rope, 0 if pairing == "halves" else 1,
                             torch.tensor(pos, dtype=torch.int32).cuda(), dec, None if norm_w is None else norm_w.cuda(), state,
                             torch.tensor(starts, dtype=torch.int32).cuda(), torch.tensor(slots, dtype=torch.int32).cuda(), heads, d,
-                            dv, INPUT_ACTIVATIONS[act], key_scale, OUTPUT_NORMS[norm_kind], GATE_ACTIVATIONS[gate], eps)
+                            dv, INPUT_ACTIVATIONS[act], key_scale, OUTPUT_NORMS[norm_kind], GATE_ACTIVATIONS[gate], eps,
+                            longest_item=max(n for _, n in step))
         at = 0
         for r, n in step:
             got[r].append(out[at : at + n].cpu())
