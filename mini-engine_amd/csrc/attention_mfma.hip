@@ -919,7 +919,7 @@ template <int D, int NB, bool MASK>
 __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, int key_base, int r, int g,
                                                 const float4_t (&s)[NB][4], const int (&qpos)[NB], const int (&lo_col)[NB],
                                                 float scale_log2, float (&m)[NB], float (&lsum)[NB],
-                                                float4_t (&acc)[NB][D / 16]) {
+                                                float4_t (&acc)[NB][D / 16], int keep_first) {
   using L = PrefillLds<D>;
   bf16x8_t pf[NB][2];
 #pragma unroll
@@ -933,7 +933,7 @@ __device__ __forceinline__ void pf_softmax_pv64(const bf16_t* __restrict__ vs, i
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const int key = key_base + (i >> 3) * 32 + g * 8 + ((i >> 2) & 1) * 4 + (i & 3);  // score tile i / 4, row 4g + i % 4
-        if (key < lo_col[nb] || key > qpos[nb]) sv[i] = -INFINITY;
+        if ((key < lo_col[nb] && key >= keep_first) || key > qpos[nb]) sv[i] = -INFINITY;  // (kept first keys stay visible)
       }
     }
     // statistics are kept in units of the raw score times scale*log2(e): one fused multiply-add per
@@ -1008,7 +1008,7 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const PrefillWork* __restrict__ work, const int* __restrict__ bundle_first, const int* __restrict__ block_table,
     int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks,
-    int nh, int nkv, int bs_shift, int window, float scale_log2, int tokens_per_block) {
+    int nh, int nkv, int bs_shift, int window, float scale_log2, int tokens_per_block, int keep_first) {
   constexpr int THREADS = WAVES * 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
@@ -1089,9 +1089,9 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     if (active) {
       const bool need_mask = key0 + PF_KT - 1 > wave_min_pos || window > 0;
       if (need_mask)
-        pf_softmax_pv64<D, NB, true>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc);
+        pf_softmax_pv64<D, NB, true>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep_first);
       else
-        pf_softmax_pv64<D, NB, false>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc);
+        pf_softmax_pv64<D, NB, false>(vs, key0, r, g, s, qpos, lo_col, scale_log2, m, lsum, acc, keep_first);
     }
     __syncthreads();
   }
@@ -1182,7 +1182,7 @@ template <int D, int NB>
 static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const PrefillWork* work,
                           const int* bundle_first, const int* table, int width, bf16_t* out,
                           float* part_o, float* part_ml, int max_chunks, int nh, int nkv, int bs_shift, int window,
-                          float sl, int tpb, hipStream_t stream) {
+                          float sl, int tpb, int keep_first, hipStream_t stream) {
   static bool configured = false;  // raise the dynamic LDS limit of this instantiation once
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, NB, PF_WAVES>),
@@ -1192,7 +1192,8 @@ static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf
     configured = true;
   }
   attention_prefill_kernel<D, NB, PF_WAVES><<<grid, PF_WAVES * 64, PrefillLds<D>::BYTES, stream>>>(
-      q, kc, vc, work, bundle_first, table, width, out, part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb);
+      q, kc, vc, work, bundle_first, table, width, out, part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb,
+      keep_first);
   return 0;
 }
 
@@ -1204,12 +1205,17 @@ static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf
 // head. When a tile's keys are cut into chunks (max_chunks > 1), part_o float [T, nh, max_chunks, d] and
 // part_ml float [T, nh, max_chunks, 2] take the partial results and token_chunks int [T] says how many
 // chunks each token's tile has (1: in one piece).
-extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, int num_items,
-                                         const int* block_table, int table_width, void* out, const int* work,
-                                         const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
-                                         const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
-                                         int d, int bs, int window, float scale, int columns, hipStream_t stream) {
+// keep_first: with a window, the keys 0 .. keep_first-1 stay visible behind it; the work list then gives a tile whose
+// window has left them behind an entry of its own for them (so such a tile always has chunks).
+extern "C" int me_attention_prefill_bf16_kept(const void* q, const void* k_cache, const void* v_cache, int num_items,
+                                              const int* block_table, int table_width, void* out, const int* work,
+                                              const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
+                                              const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
+                                              int d, int bs, int window, int keep_first, float scale, int columns,
+                                              hipStream_t stream) {
   const int num_work = num_bundles;
+  if (keep_first < 0 || (keep_first > 0 && window <= 0))
+    return me_fail("me_attention_prefill_bf16: keep_first=%d needs a window", keep_first);
   if (num_items <= 0 || num_work <= 0) return 0;
   if (!me_attention_mfma_supported(d, bs))
     return me_fail("me_attention_prefill_bf16: head_dim=%d / block_size=%d not supported by the matrix-core kernels", d, bs);
@@ -1237,10 +1243,10 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
   case DD:                                                                                                         \
     rc = wide ? launch_prefill<DD, 2>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table,       \
                                       table_width, (bf16_t*)out, part_o, part_ml, max_chunks, nh, nkv, bs_shift,   \
-                                      window, sl, tpb, stream)                                                     \
+                                      window, sl, tpb, keep_first, stream)                                         \
               : launch_prefill<DD, 1>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table,       \
                                       table_width, (bf16_t*)out, part_o, part_ml, max_chunks, nh, nkv, bs_shift,   \
-                                      window, sl, tpb, stream);                                                    \
+                                      window, sl, tpb, keep_first, stream);                                        \
     break;
   switch (d) {
     ME_PREFILL_CASE(32)
@@ -1259,6 +1265,16 @@ extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, con
     return me_check_launch("me_attention_prefill_combine");
   }
   return 0;
+}
+
+extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, int num_items,
+                                         const int* block_table, int table_width, void* out, const int* work,
+                                         const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
+                                         const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
+                                         int d, int bs, int window, float scale, int columns, hipStream_t stream) {
+  return me_attention_prefill_bf16_kept(q, k_cache, v_cache, num_items, block_table, table_width, out, work, bundle_first,
+                                        num_bundles, part_o, part_ml, token_chunks, max_chunks, num_tokens, nh, nkv, d, bs, window,
+                                        0, scale, columns, stream);
 }
 
 // ------------------------------------------------------------------------------------ the splits' sum inside the output projection

@@ -978,3 +978,39 @@ extern "C" int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const fl
         (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, dv, bs, eps, hpb);
   return me_check_launch("me_qkv_rotate_scatter");
 }
+
+// ---------------------------------------------------------------- rows turned back by their positions' angles
+// rows [T, heads, n] in place: pair j of every head, (j, j + n/2) with pairing 0 and (2j, 2j + 1) with pairing 1, by
+// minus the angle j of the token's position: (u, v) -> (u cos + v sin, v cos - u sin). table float32 [positions, 2, n/2].
+// What attention over values that were turned by their own positions owes its outputs.
+template <typename T>
+__global__ void unturn_rows_kernel(T* __restrict__ rows, const float* __restrict__ table, int pairing,
+                                   const int* __restrict__ positions, int heads, int n, size_t pairs) {
+  const int half = n / 2;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < pairs; i += (size_t)gridDim.x * blockDim.x) {
+    const int j = (int)(i % half);
+    const size_t th = i / half;  // token * heads + head
+    const int t = (int)(th / heads);
+    const float* cs = table + (size_t)positions[t] * n;
+    const float c = cs[j], sn = cs[half + j];
+    T* row = rows + th * n;
+    const int a = pairing == 0 ? j : 2 * j, b = pairing == 0 ? j + half : 2 * j + 1;
+    const float u = to_float(row[a]), v = to_float(row[b]);
+    row[a] = from_float<T>(u * c + v * sn);
+    row[b] = from_float<T>(v * c - u * sn);
+  }
+}
+
+extern "C" int me_unturn_rows(void* rows, const float* table, int pairing, const int* positions, int num_tokens, int heads, int n,
+                              int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads <= 0 || n <= 0 || n % 2 || (pairing & ~1)) return me_fail("me_unturn_rows: heads=%d n=%d pairing=%d", heads, n, pairing);
+  const size_t pairs = (size_t)num_tokens * heads * (n / 2);
+  const size_t want = (pairs + 255) / 256;
+  const int blocks = (int)(want < 8192 ? want : 8192);
+  if (dtype == ME_F32)
+    unturn_rows_kernel<float><<<blocks, 256, 0, stream>>>((float*)rows, table, pairing, positions, heads, n, pairs);
+  else
+    unturn_rows_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)rows, table, pairing, positions, heads, n, pairs);
+  return me_check_launch("me_unturn_rows");
+}

@@ -19,6 +19,8 @@ constexpr long long kPartialBytesMax = 256ll << 20;  // most memory the partial 
 
 struct Tile {
   int item, first_token, tokens, first_pos, first_key, last_pos, key_tiles;
+  int kept_tiles = 0;  // key tiles of the kept first keys that the tile's window has left behind: they come before the window's
+                       // in the tile's order of key tiles, and lie at keys 0 .. 64 * kept_tiles - 1
 };
 struct Piece {
   int length, tile, chunk, first_tile;  // chunk -1: the tile in one piece
@@ -29,13 +31,14 @@ struct Piece {
 std::vector<Piece> cut(const std::vector<Tile>& tiles, int cap) {
   std::vector<Piece> pieces;
   for (int i = 0; i < (int)tiles.size(); ++i) {
-    const int n = tiles[i].key_tiles;
-    if (n <= cap) {
+    const int n = tiles[i].key_tiles, kept = tiles[i].kept_tiles;
+    if (kept == 0 && n <= cap) {
       pieces.push_back({n, i, -1, 0});
       continue;
     }
-    int j = 0;
-    for (int t0 = 0; t0 < n; t0 += cap, ++j) pieces.push_back({std::min(cap, n - t0), i, j, t0});
+    int j = 0;  // (no piece reaches across the gap between the kept keys and the window)
+    for (int t0 = 0; t0 < kept; t0 += cap, ++j) pieces.push_back({std::min(cap, kept - t0), i, j, t0});
+    for (int t0 = 0; t0 < n; t0 += cap, ++j) pieces.push_back({std::min(cap, n - t0), i, j, kept + t0});
   }
   return pieces;
 }
@@ -97,7 +100,7 @@ bool wide_blocks_pay(const int* starts, const int* qlens, int items, int tpb, in
 // results a second kernel adds up, and the pieces are packed into one bundle per compute unit; `cap` is
 // the candidate with the shortest longest bundle, where cutting at all counts as kCutOverhead key tiles.
 void build_work_list(const int* starts, const int* qlens, int items, int tpb, int window, int nkv, int slots,
-                     long long partial_row_bytes, WorkList& out) {
+                     long long partial_row_bytes, WorkList& out, int keep_first) {
   std::vector<Tile> tiles;
   int offset = 0;
   for (int i = 0; i < items; ++i) {
@@ -106,6 +109,7 @@ void build_work_list(const int* starts, const int* qlens, int items, int tpb, in
       const int p_first = starts[i] + t0, p_last = p_first + count - 1;
       const int k0 = window > 0 ? (std::max(p_first - window + 1, 0) / 64) * 64 : 0;
       tiles.push_back({i, offset + t0, count, p_first, k0, p_last, (p_last - k0) / 64 + 1});
+      if (window > 0 && keep_first > 0 && k0 > 0) tiles.back().kept_tiles = (std::min(keep_first, k0) + 63) / 64;
     }
     offset += qlens[i];
   }
@@ -113,8 +117,8 @@ void build_work_list(const int* starts, const int* qlens, int items, int tpb, in
   int longest = 0;
   long long total = 0;
   for (const Tile& t : tiles) {
-    longest = std::max(longest, t.key_tiles);
-    total += t.key_tiles;
+    longest = std::max(longest, t.key_tiles + t.kept_tiles);
+    total += t.key_tiles + t.kept_tiles;
   }
   std::vector<std::vector<Piece>> bundles;
   if ((int)tiles.size() > bins) {
@@ -124,6 +128,7 @@ void build_work_list(const int* starts, const int* qlens, int items, int tpb, in
   } else {
     long long chunk_limit = 1ll << 30;
     if (partial_row_bytes > 0) chunk_limit = std::max(1ll, kPartialBytesMax / (partial_row_bytes * std::max(1, offset)));
+    if (keep_first > 0) chunk_limit = std::max(1ll, chunk_limit - 1);  // (the kept keys' piece is one more)
     std::vector<int> caps = {longest, (int)((total + bins - 1) / bins), (int)((total + 2ll * bins - 1) / (2ll * bins)),
                              (longest + 1) / 2, (longest + 2) / 3};
     std::sort(caps.begin(), caps.end());
@@ -164,8 +169,10 @@ void build_work_list(const int* starts, const int* qlens, int items, int tpb, in
     out.bundle_first.push_back((int)out.work.size() / 8);
     for (const Piece& p : bundle) {
       const Tile& t = tiles[p.tile];
-      const int row[8] = {t.item, t.first_token, t.tokens, t.first_pos, t.first_key + 64 * p.first_tile,
-                          std::min(t.last_pos, t.first_key + 64 * (p.first_tile + p.length) - 1), p.chunk, 0};
+      const bool of_kept = p.first_tile < t.kept_tiles;
+      const int begin = of_kept ? 64 * p.first_tile : t.first_key + 64 * (p.first_tile - t.kept_tiles);
+      const int row[8] = {t.item, t.first_token, t.tokens, t.first_pos, begin,
+                          std::min(of_kept ? std::min(keep_first, t.first_key) - 1 : t.last_pos, begin + 64 * p.length - 1), p.chunk, 0};
       out.work.insert(out.work.end(), row, row + 8);
     }
     out.work.back() = 1;  // the bundle ends with this entry
@@ -186,11 +193,12 @@ extern "C" {
 // For Python callers and tests: the work list as flat arrays. work takes 8 ints per entry, bundle_first one per
 // bundle, token_chunks one per token; counts: entries, bundles, max chunks. Returns 0, or -1 when a buffer is
 // too small (counts then say what is needed).
-int me_prefill_work_list(const int32_t* starts, const int32_t* qlens, int items, int tpb, int window, int nkv, int slots,
-                         long long partial_row_bytes, int32_t* work, int cap_entries, int32_t* bundle_first, int cap_bundles,
-                         int32_t* token_chunks, int cap_tokens, int32_t* counts) {
+// keep_first: with a window, the first keys that stay visible behind it (an entry of their own per tile that has left them).
+int me_prefill_work_list_kept(const int32_t* starts, const int32_t* qlens, int items, int tpb, int window, int keep_first, int nkv,
+                              int slots, long long partial_row_bytes, int32_t* work, int cap_entries, int32_t* bundle_first,
+                              int cap_bundles, int32_t* token_chunks, int cap_tokens, int32_t* counts) {
   me::WorkList list;
-  me::build_work_list(starts, qlens, items, tpb, window, nkv, slots, partial_row_bytes, list);
+  me::build_work_list(starts, qlens, items, tpb, window, nkv, slots, partial_row_bytes, list, keep_first);
   counts[0] = (int)list.work.size() / 8;
   counts[1] = (int)list.bundle_first.size();
   counts[2] = list.max_chunks;
@@ -199,6 +207,13 @@ int me_prefill_work_list(const int32_t* starts, const int32_t* qlens, int items,
   std::copy(list.bundle_first.begin(), list.bundle_first.end(), bundle_first);
   std::copy(list.token_chunks.begin(), list.token_chunks.end(), token_chunks);
   return 0;
+}
+
+int me_prefill_work_list(const int32_t* starts, const int32_t* qlens, int items, int tpb, int window, int nkv, int slots,
+                         long long partial_row_bytes, int32_t* work, int cap_entries, int32_t* bundle_first, int cap_bundles,
+                         int32_t* token_chunks, int cap_tokens, int32_t* counts) {
+  return me_prefill_work_list_kept(starts, qlens, items, tpb, window, 0, nkv, slots, partial_row_bytes, work, cap_entries,
+                                   bundle_first, cap_bundles, token_chunks, cap_tokens, counts);
 }
 
 // The two limits of wide_blocks_pay (blocks and key tiles per compute unit), for measurements and tests that

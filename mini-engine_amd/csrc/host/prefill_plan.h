@@ -17,6 +17,6 @@ struct WorkList {
 
 bool wide_blocks_pay(const int* starts, const int* qlens, int items, int tpb, int window, int nkv, int slots);
 void build_work_list(const int* starts, const int* qlens, int items, int tpb, int window, int nkv, int slots,
-                     long long partial_row_bytes, WorkList& out);
+                     long long partial_row_bytes, WorkList& out, int keep_first = 0);
 
 }  // namespace me

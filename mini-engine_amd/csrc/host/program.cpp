@@ -143,6 +143,13 @@ bool attention_is_plain(const Op& op) {
   return (op.i[9] == 0 || op.i[9] == op.i[2]) && op.i[10] == 0 && op.i[11] == 0 && op.i[12] == 0;
 }
 
+// Whether prompts of an attention operation beyond the plain form go to the tiled matrix-core kernel: bfloat16, keys and
+// values of one size that the kernel is built for, up to 16 heads to a key/value head.
+bool attention_takes_tiled_prefill(const Op& op, int dtype) {
+  const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], bs = (int)op.i[4];
+  return dtype == kBF16 && (op.i[9] == 0 || op.i[9] == d) && me_attention_mfma_supported(d, bs) && nh / nkv <= 16;
+}
+
 int groups_of(int64_t v) { return v > 1 ? (int)v : 1; }
 float scale_of(float f) { return f == 0.f ? 1.f : f; }
 
@@ -431,6 +438,23 @@ class Run {
       void* q = arena_.take((size_t)t_ * nh * d * elem_);
       ok(me_qkv_rotate_scatter(qkv, q_w, k_w, rope, rd, pairing, v_table, v_pairing, idx(s_.lay.positions), idx(s_.lay.token_item),
                                table, width, q, kc, vc, t_, nh, nkv, d, dv, bs, eps, dtype_, stream_));
+      if (!s_.decode_only && attention_takes_tiled_prefill(op, dtype_)) {
+        // prompts and portions in bfloat16 with keys and values of one size the matrix cores take: the tiled kernel, whose
+        // work list has an entry of its own for the kept first keys; the outputs are turned back by a pass of their own
+        auto it = s_.plans.find({nh, nkv, d, window, keep_first});
+        if (it == s_.plans.end()) throw Error(kBroken, "the step has no work list for a prefill attention layer");
+        const StepView::Plan& p = it->second;
+        float *part_o = nullptr, *part_ml = nullptr;
+        if (p.max_chunks > 1) {
+          part_o = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * d * 4);
+          part_ml = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * 2 * 4);
+        }
+        ok(me_attention_prefill_bf16_kept(q, kc, vc, items, table, width, out, idx(p.work), idx(p.bundle_first), p.bundles, part_o,
+                                          part_ml, p.token_chunks >= 0 ? idx(p.token_chunks) : nullptr, p.max_chunks, t_, nh, nkv, d,
+                                          bs, window, keep_first, scale, p.columns, stream_));
+        if (v_table) ok(me_unturn_rows(out, v_table, v_pairing, idx(s_.lay.positions), t_, nh, dv, dtype_, stream_));
+        return;
+      }
       ok(me_attention_general_ext(q, kc, vc, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, out, t_, nh, nkv, d, dv, bs,
                                   window, keep_first, v_table, v_pairing, scale, dtype_, items, stream_));
       return;
@@ -493,7 +517,7 @@ class Run {
       return;
     }
     if (mfma) {
-      auto it = s_.plans.find({nh, nkv, d, window});
+      auto it = s_.plans.find({nh, nkv, d, window, 0});
       if (it == s_.plans.end()) throw Error(kBroken, "the step has no work list for a prefill attention layer");
       const StepView::Plan& p = it->second;
       float *part_o = nullptr, *part_ml = nullptr;
@@ -622,10 +646,11 @@ std::vector<std::vector<int>> Program::prefill_geometries() const {
   std::vector<std::vector<int>> out;
   if (dtype_ != kBF16) return out;
   for (const Op& op : ops_) {
-    if (op.kind != kOpAttention || !attention_is_plain(op)) continue;
+    if (op.kind != kOpAttention) continue;
     const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], bs = (int)op.i[4], window = (int)op.i[5];
+    if (!attention_is_plain(op) && !attention_takes_tiled_prefill(op, dtype_)) continue;
     if (!me_attention_mfma_supported(d, bs) || nh / nkv > 16) continue;
-    std::vector<int> key = {nh, nkv, d, window};
+    std::vector<int> key = {nh, nkv, d, window, attention_is_plain(op) ? 0 : (int)op.i[10]};
     if (std::find(out.begin(), out.end(), key) == out.end()) out.push_back(key);
   }
   return out;
@@ -646,6 +671,9 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
       need = (size_t)me_decay_state_workspace(tokens, items, (int)op.i[0], (int)op.i[1], (int)op.i[2]) + pad;
     if (op.kind == kOpAttention && !attention_is_plain(op)) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
+      if (attention_takes_tiled_prefill(op, dtype_) && tokens > items)  // partial results of cut tiles: the work list's bound,
+        need += (size_t)(256ll << 20) + (size_t)(256ll << 20) * 2 / op.i[2] +  // and one chunk more for the kept first keys
+                (size_t)tokens * op.i[0] * (op.i[2] + 2) * 4 * 2 + 2 * pad;
     } else if (op.kind == kOpAttention) {
       const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2];
       const int chunks = (nh / nkv + 15) / 16;

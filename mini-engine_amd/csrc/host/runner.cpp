@@ -66,7 +66,7 @@ void hip_ok(hipError_t e, const char* what) {
 
 // The work list of one attention geometry for the current step, from the cache or made now.
 const CachedPlan& plan_for(Runner& r, const std::vector<int>& geometry) {
-  const int nh = geometry[0], nkv = geometry[1], d = geometry[2], window = geometry[3];
+  const int nh = geometry[0], nkv = geometry[1], d = geometry[2], window = geometry[3], keep_first = geometry[4];
   std::vector<int> key = geometry;
   key.insert(key.end(), r.starts.begin(), r.starts.end());
   key.push_back(-1);
@@ -83,7 +83,7 @@ const CachedPlan& plan_for(Runner& r, const std::vector<int>& geometry) {
                                         std::max(1, me_attention_prefill_columns(1) / group), window, nkv, r.compute_units);
   fresh.columns = me_attention_prefill_columns(wide ? 1 : 0);
   me::build_work_list(r.starts.data(), r.qlens.data(), items, fresh.columns / group, window, nkv, r.compute_units,
-                      (long long)nh * d * 4, fresh.list);
+                      (long long)nh * d * 4, fresh.list, keep_first);
   r.plans.push_front(std::move(fresh));
   if (r.plans.size() > 64) r.plans.pop_back();
   return r.plans.front();
@@ -138,7 +138,7 @@ int64_t me_runner_index_need(void* runner, int tokens, int items, int rows, cons
                const me::StepLayout l = me::StepLayout::make(tokens, items, rows, std::vector<int>(widths, widths + num_groups));
                // tiles: at most one per 1 token-run of an item plus one per item; cut pieces: at most as many again
                // plus two per compute unit; 8 ints per entry, one per bundle, one per token
-               const int64_t entries = 2 * ((int64_t)tokens / 4 + items) + 2048;
+               const int64_t entries = 3 * ((int64_t)tokens / 4 + items) + 2048;  // (and one per tile for kept first keys)
                return (int64_t)l.total + (int64_t)r->geometries.size() * (entries * 9 + tokens) + 64;)
 }
 

@@ -71,6 +71,13 @@ int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_
                               int table_width, void* out, const int* work, const int* bundle_first, int num_bundles,
                               float* part_o, float* part_ml, const int* token_chunks, int max_chunks, int num_tokens, int nh,
                               int nkv, int d, int bs, int window, float scale, int columns, hipStream_t stream);
+int me_attention_prefill_bf16_kept(const void* q, const void* k_cache, const void* v_cache, int num_items, const int* block_table,
+                                   int table_width, void* out, const int* work, const int* bundle_first, int num_bundles,
+                                   float* part_o, float* part_ml, const int* token_chunks, int max_chunks, int num_tokens,
+                                   int nh, int nkv, int d, int bs, int window, int keep_first, float scale, int columns,
+                                   hipStream_t stream);
+int me_unturn_rows(void* rows, const float* table, int pairing, const int* positions, int num_tokens, int heads, int n,
+                   int dtype, hipStream_t stream);
 int me_gemm_f32(const float* A, const float* W, float* C, int M, int N, int K, hipStream_t stream);
 int me_gemm_plain(const void* A, const void* W, void* C, int M, int N, int K, int in_dtype, int out_dtype, hipStream_t stream);
 int me_gemm_bf16_small(const void* X, const float* x_in, const void* delta, const float* w_norm, float eps, float* x_out,

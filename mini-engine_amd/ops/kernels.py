@@ -1038,7 +1038,7 @@ class PrefillPlan:
 
 
 def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int, nkv: int, slots: int,
-                      partial_row_bytes: int = 0):
+                      partial_row_bytes: int = 0, keep_first: int = 0):
     """Host side of :class:`PrefillPlan`: (entries int32 [n, 8], first entry of each bundle int32 [b],
     chunks per token int32 [T], max chunks), as ``csrc/host/prefill_plan.cpp`` builds it (the native
     step uses the same builder).
@@ -1047,7 +1047,8 @@ def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int
     multiple of 64) to its last token's position. A bundle of entries is run by one block per kv head;
     tiles of a step with few of them are cut into key ranges whose partial results a second kernel adds
     up. An entry is (item, first token, tokens, first position, first key, last key, chunk or -1, 1 if
-    its bundle ends with it)."""
+    its bundle ends with it). With ``keep_first`` (and a window) a tile whose window has left the first keys behind
+    has an entry of its own for the keys ``0 .. min(keep_first, its window's first tile) - 1``, so it always has chunks."""
     s = np.ascontiguousarray(starts, dtype=np.int32)
     q = np.ascontiguousarray(qlens, dtype=np.int32)
     total = int(q.sum())
@@ -1057,10 +1058,10 @@ def prefill_work_list(starts: list[int], qlens: list[int], tpb: int, window: int
         work = np.empty((cap_entries, 8), dtype=np.int32)
         first = np.empty(cap_bundles, dtype=np.int32)
         token_chunks = np.empty(total, dtype=np.int32)
-        rc = lib().me_prefill_work_list(_vp(s.ctypes.data), _vp(q.ctypes.data), _i(len(q)), _i(tpb), _i(window), _i(nkv),
-                                        _i(slots), ctypes.c_longlong(partial_row_bytes), _vp(work.ctypes.data), _i(cap_entries),
-                                        _vp(first.ctypes.data), _i(cap_bundles), _vp(token_chunks.ctypes.data), _i(total),
-                                        _vp(counts.ctypes.data))
+        rc = lib().me_prefill_work_list_kept(_vp(s.ctypes.data), _vp(q.ctypes.data), _i(len(q)), _i(tpb), _i(window),
+                                             _i(keep_first), _i(nkv), _i(slots), ctypes.c_longlong(partial_row_bytes),
+                                             _vp(work.ctypes.data), _i(cap_entries), _vp(first.ctypes.data), _i(cap_bundles),
+                                             _vp(token_chunks.ctypes.data), _i(total), _vp(counts.ctypes.data))
         if rc == 0:
             return work, first, token_chunks, int(counts[2])
         cap_entries, cap_bundles = int(counts[0]), int(counts[1])
@@ -1071,14 +1072,14 @@ _PLANS: dict = {}  # the last plans made, by what they were made from: steps of 
 
 
 def prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device,
-                 wide: bool | None = None) -> PrefillPlan:
+                 wide: bool | None = None, keep_first: int = 0) -> PrefillPlan:
     """``wide``: blocks of twice as many query columns or not; None lets the step's size decide."""
-    key = (tuple(starts), tuple(qlens), nh, nkv, d, window, str(device), wide)
+    key = (tuple(starts), tuple(qlens), nh, nkv, d, window, str(device), wide, keep_first)
     plan = _PLANS.get(key)
     if plan is None:
         if len(_PLANS) >= 64:
             _PLANS.pop(next(iter(_PLANS)))
-        plan = _PLANS[key] = _make_prefill_plan(starts, qlens, nh, nkv, d, window, device, wide)
+        plan = _PLANS[key] = _make_prefill_plan(starts, qlens, nh, nkv, d, window, device, wide, keep_first)
     return plan
 
 
@@ -1103,14 +1104,14 @@ def set_prefill_wide_limits(min_blocks: float, min_key_tiles: float) -> tuple[fl
 
 
 def _make_prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d: int, window: int, device,
-                       wide: bool | None = None) -> PrefillPlan:
+                       wide: bool | None = None, keep_first: int = 0) -> PrefillPlan:
     group = nh // nkv
     slots = torch.cuda.get_device_properties(device).multi_processor_count
     if wide is None:
         wide = wide_blocks_pay(starts, qlens, max(1, lib().me_attention_prefill_columns(1) // group), window, nkv, slots)
     columns = lib().me_attention_prefill_columns(1 if wide else 0)
     tpb = columns // group
-    work, first, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, nh * d * 4)
+    work, first, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, nh * d * 4, keep_first)
     parts = [work.reshape(-1), first] + ([token_chunks] if max_chunks > 1 else [])
     both = torch.from_numpy(np.concatenate(parts)).to(device)  # one upload
     a, b = work.size, work.size + first.size
@@ -1119,12 +1120,13 @@ def _make_prefill_plan(starts: list[int], qlens: list[int], nh: int, nkv: int, d
 
 def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: list[int], block_table, scale: float,
                            window: int = 0, out: torch.Tensor | None = None, starts: list[int] | None = None,
-                           plan: PrefillPlan | None = None) -> torch.Tensor:
+                           plan: PrefillPlan | None = None, keep_first: int = 0) -> torch.Tensor:
     """Causal attention of packed new tokens q [T, nh, d] bfloat16 over the paged cache (which already
     holds the new tokens' keys and values). item_start int32 [items + 1] are the items' offsets into
     the packed tokens, ``qlens`` the same lengths on the host and ``starts`` the position of each item's
     first token (read back from ``positions`` when not given); ``plan`` is what :func:`prefill_plan`
-    makes of them, for callers that run several layers on one step."""
+    makes of them, for callers that run several layers on one step (made with the same ``keep_first``: the first
+    keys that stay visible behind the window)."""
     _want(q, "q", torch.bfloat16, (None, None, None))
     t, nh, d = q.shape
     nkv, bs = k_cache.shape[1], k_cache.shape[2]
@@ -1142,7 +1144,7 @@ def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: li
         if starts is None:
             firsts = np.concatenate([[0], np.cumsum(qlens)[:-1]])
             starts = positions[torch.from_numpy(firsts).to(positions.device)].tolist()
-        plan = prefill_plan(starts, qlens, nh, nkv, d, window, q.device)
+        plan = prefill_plan(starts, qlens, nh, nkv, d, window, q.device, keep_first=keep_first)
     if out is None:
         out = torch.empty((t, nh * d), dtype=torch.bfloat16, device=q.device)
     _want(out, "out", torch.bfloat16, (t, nh * d))
@@ -1150,10 +1152,22 @@ def attention_prefill_bf16(q, k_cache, v_cache, positions, item_start, qlens: li
     if plan.max_chunks > 1:
         part_o = torch.empty((t * nh * plan.max_chunks * d,), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((t * nh * plan.max_chunks * 2,), dtype=torch.float32, device=q.device)
-    check(lib().me_attention_prefill_bf16(
+    check(lib().me_attention_prefill_bf16_kept(
         _p(q), _p(k_cache), _p(v_cache), _i(items), _p(block_table),
         _i(block_table.shape[1]), _p(out), _p(plan.work), _p(plan.bundle_first), _i(plan.num_bundles), _p(part_o), _p(part_ml),
-        _p(plan.token_chunks), _i(plan.max_chunks), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale),
+        _p(plan.token_chunks), _i(plan.max_chunks), _i(t), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _i(keep_first), _f(scale),
         _i(plan.columns), _stream()))
     return out
+
+
+def unturn_rows(rows: torch.Tensor, table: torch.Tensor, pairing: int, positions: torch.Tensor, heads: int) -> torch.Tensor:
+    """``rows`` ``[T, heads * n]`` in place: every head's pairs turned back by the angles of the token's position
+    (``table`` float32 ``[P, 2, n / 2]``; pairing 0: j with j + n/2, 1: 2j with 2j + 1)."""
+    _want(rows, "rows", None, (None, None))
+    t, n = rows.shape[0], rows.shape[1] // heads
+    _want(table, "table", torch.float32, (None, 2, n // 2))
+    _want(positions, "positions", torch.int32, (t,))
+    check(lib().me_unturn_rows(_p(rows), _p(table), _i(pairing), _p(positions), _i(t), _i(heads), _i(n), _i(_code(rows.dtype)),
+                               _stream()))
+    return rows
 

@@ -126,6 +126,20 @@ class Attention(Mixer):
             v_pairing = 0 if self.value_position is None else self.value_position.pairing_code
             q = K.qkv_rotate_scatter(proj, self.q_norm_w, self.k_norm_w, rope, self.pairing, vt, v_pairing, batch.positions,
                                      batch.token_item, table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, self.dv, eps)
+            if (self.dtype is torch.bfloat16 and not batch.decode_only and self.dv == self.d
+                    and K.attention_mfma_supported(self.d, b.block_size, self.nh // self.nkv)):
+                # prompts and portions: the tiled matrix-core kernel, then the outputs turned back in a pass of their own
+                key = ("prefill_plan", self.nh, self.nkv, self.d, int(s.window), self.keep_first)
+                plan = batch.derived.get(key)
+                if plan is None:
+                    plan = K.prefill_plan(batch.starts, batch.qlens, self.nh, self.nkv, self.d, int(s.window), q.device,
+                                          keep_first=self.keep_first)
+                    batch.derived[key] = plan
+                out = K.attention_prefill_bf16(q, b.k_cache, b.v_cache, batch.positions, batch.item_start, batch.qlens, table,
+                                               float(s.scale), int(s.window), plan=plan, keep_first=self.keep_first)
+                if vt is not None:
+                    K.unturn_rows(out, vt, v_pairing, batch.positions, self.nh)
+                return K.linear(out, self.w_o, as_delta=True)
             out = K.attention_general(q, b.k_cache, b.v_cache, batch.positions, batch.token_item, table, float(s.scale),
                                       int(s.window), keep_first=self.keep_first, unturn=vt, un_pairing=v_pairing)
             return K.linear(out, self.w_o, as_delta=True)

@@ -50,10 +50,15 @@ def configs() -> dict[str, dict]:
             attention(3, 3, 24, 20, 17, 17, 24, 100.0, 0.3, ff=104),
             retention(5, 40, 12, (0.7, 0.9, 0.95, 0.99, 0.999), 20, 1e3, ff=104),
             lightning(1, 72, 136, (0.97,))]),
+        # keys and values of one size that the matrix cores take: prompts in bfloat16 run the tiled attention kernel
+        "S": model(210, 128, 2, 0.6, 1e-6, [
+            attention(4, 2, 64, 64, 50, 6, 32, 1e4, 0.125, ff=128),
+            lightning(2, 32, 32, (0.9, 0.99)),
+            attention(8, 8, 32, 32, 100, 70, 32, 1e5, 0.2, ff=128)]),
     }
 
 
-BLOCK_SIZES = {"P": 16, "Q": 32, "R": 8}
+BLOCK_SIZES = {"P": 16, "Q": 32, "R": 8, "S": 16}
 
 
 def write_folder(folder: str, cfg: dict, seed: int = 0, std: float = 0.08) -> str:

@@ -143,6 +143,62 @@ def test_window_attention_in_portions_with_one_key_that_stands_out(nh, nkv, d, d
     assert rel_err(other, want) > 0.05
 
 
+@pytest.mark.parametrize("nh,nkv,d,rd,pairing,size,keep", [(4, 2, 64, 32, "interleaved", 50, 6), (8, 8, 32, 32, "halves", 100, 70),
+                                                          (6, 1, 128, 128, "interleaved", 70, 1), (2, 1, 64, 64, "halves", 200, 130)])
+def test_tiled_prompt_attention_sees_the_kept_first_keys(nh, nkv, d, rd, pairing, size, keep):
+    """bfloat16 prompts and portions with keys and values of one size go to the tiled matrix-core kernel, whose work
+    list gives the kept first keys an entry of their own: two sequences side by side, in portions that start behind the
+    kept keys, with the same loud keys as above."""
+    from mini_engine_amd.ops import kernels as K
+
+    dtype, base, eps, scale, bs = torch.bfloat16, 500.0, 1e-5, 0.3, 16
+    g = torch.Generator().manual_seed(nh * 100 + d)
+    lens = [330, 205]
+    u = torch.randn(d, generator=g)
+    seqs, wants = [], []
+    for L in lens:
+        qkv = torch.randn(L, (nh + 2 * nkv) * d, generator=g) * 0.5
+        for j in (0, max(keep - 1, 0), keep, 63, 64, 150, L - size, L - size - 1, L - 2):
+            if 0 <= j < L:
+                qkv[j, nh * d + (j % nkv) * d : nh * d + (j % nkv + 1) * d] += 3.0 * u
+        qkv[:, : nh * d] += 0.7 * u.repeat(nh)
+        qkv = qkv.to(dtype)
+        seqs.append(qkv)
+        wants.append(plain_attention_rows(qkv.float(), 0, nh, nkv, d, d, None, None, eps, rd, base, pairing, True, scale, size, keep))
+    pages = [-(-L // bs) for L in lens]
+    order = torch.randperm(sum(pages) + 2, generator=g).to(torch.int32)
+    table = torch.full((2, max(pages)), int(order[-1]), dtype=torch.int32)
+    table[0, : pages[0]] = order[: pages[0]]
+    table[1, : pages[1]] = order[pages[0] : pages[0] + pages[1]]
+    table = table.cuda()
+    k_cache = torch.zeros(sum(pages) + 2, nkv, bs, d, dtype=dtype, device="cuda")
+    v_cache = torch.zeros(sum(pages) + 2, nkv, d, bs, dtype=dtype, device="cuda")
+    rope, vt = angle_table(rd, base, 512), angle_table(d, base, 512)
+    code = 0 if pairing == "halves" else 1
+    got = [[], []]
+    for cuts in ([(0, 130), (0, 5)], [(130, 331 - 1), (5, 205)]):
+        qlens = [hi - lo for lo, hi in cuts]
+        starts = [lo for lo, _ in cuts]
+        pos = torch.cat([torch.arange(lo, hi) for lo, hi in cuts]).to(torch.int32).cuda()
+        item = torch.cat([torch.full((n,), i) for i, n in enumerate(qlens)]).to(torch.int32).cuda()
+        item_start = torch.tensor([0, qlens[0], sum(qlens)], dtype=torch.int32).cuda()
+        rows = torch.cat([seqs[i][lo:hi] for i, (lo, hi) in enumerate(cuts)]).cuda().contiguous()
+        q = K.qkv_rotate_scatter(rows, None, None, rope, code, vt, code, pos, item, table, k_cache, v_cache, nh, nkv, d, d, eps)
+        out = K.attention_prefill_bf16(q, k_cache, v_cache, pos, item_start, qlens, table, scale, size, starts=starts,
+                                       keep_first=keep)
+        K.unturn_rows(out, vt, code, pos, nh)
+        got[0].append(out[: qlens[0]].cpu())
+        got[1].append(out[qlens[0] :].cpu())
+        # the kernel that takes every size, on the same pages: the two differ by the rounding of the weights alone
+        same = K.attention_general(q, k_cache, v_cache, pos, item, table, scale, size, keep_first=keep, unturn=vt, un_pairing=code)
+        assert rel_err(out, same) < 2e-2
+    for i in range(2):
+        # (scores this loud feel the rounding of the turned q and k: both kernels are up to 6% of a row's largest value off)
+        assert rel_err(torch.cat(got[i]), wants[i]) < 8e-2
+    missed = plain_attention_rows(seqs[0].float(), 0, nh, nkv, d, d, None, None, eps, rd, base, pairing, True, scale, size, 0)
+    assert rel_err(missed, wants[0]) > 0.1  # without the kept keys the longer sequence's rows are somewhere else
+
+
 # ------------------------------------------------------------------------------------------ decay state
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("heads,d,dv,rd,pairing,act,norm_kind,gate", [
@@ -251,7 +307,7 @@ def requests_for(cfg, seed, lengths=(1, 23, 97, 150, 61)):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q", "R"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
 def test_every_way_of_cutting_gives_the_plain_logits(folders, name, dtype):
     """Whole prompts; most of a prompt and its tail token by token (replayed graphs); portions down to two tokens; up
     to four live requests in a pool and in slots that are used again: all against the plain implementation."""

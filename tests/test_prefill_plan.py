@@ -100,3 +100,38 @@ def test_wide_blocks_are_taken_for_full_steps_and_long_contexts_only():
     assert pay([8192] * 2, [512] * 2)
     assert not pay([0] * 64, [64] * 64)    # wide blocks would be half empty
     assert not pay([8192] * 2, [512] * 2, window=256)  # a window takes the long walk away
+
+
+def test_kept_first_keys_get_an_entry_of_their_own_once_the_window_has_left_them():
+    """Every (token tile, key) pair that the window with kept first keys lets through lies in exactly one entry's range,
+    and entries hold no key tile that the tile cannot see at all."""
+    rng = random.Random(4)
+    for _ in range(40):
+        items = rng.randint(1, 4)
+        starts = [rng.choice([0, 0, 5, 64, 200, 1000]) for _ in range(items)]
+        qlens = [rng.choice([1, 7, 64, 130, 700]) for _ in range(items)]
+        tpb, window, keep = rng.choice([8, 64]), rng.choice([16, 100, 1024]), rng.choice([1, 4, 64, 70, 300])
+        nkv, slots = rng.choice([1, 8]), rng.choice([8, 256])
+        work, first, token_chunks, max_chunks = prefill_work_list(starts, qlens, tpb, window, nkv, slots, partial_row_bytes=4096,
+                                                                  keep_first=keep)
+        by_tile = {}
+        for item, tb, count, p_first, k0, k_last, chunk, last in work.tolist():
+            assert k0 % 64 == 0 and k0 <= k_last
+            by_tile.setdefault((item, tb, count, p_first), []).append((chunk, k0, k_last))
+        offsets = np.concatenate([[0], np.cumsum(qlens)])
+        want_tiles = {(i, int(offsets[i]) + t * tpb, min(tpb, n - t * tpb), s0 + t * tpb)
+                      for i, (s0, n) in enumerate(zip(starts, qlens)) for t in range(-(-n // tpb))}
+        assert set(by_tile) == want_tiles
+        for (item, tb, count, p_first), pieces in by_tile.items():
+            p_last = p_first + count - 1
+            covered = [k for _, a, b in pieces for k in range(a, b + 1)]
+            assert len(covered) == len(set(covered))  # no key twice
+            seen = {k for p in range(p_first, p_last + 1) for k in range(p + 1) if p - k < window or k < keep}
+            assert seen <= set(covered)
+            for _, a, b in pieces:  # every entry holds a key that some token of the tile sees
+                assert any(k in seen for k in range(a, b + 1))
+            if len(pieces) == 1:
+                assert pieces[0][0] == -1 and (token_chunks[tb:tb + count] == 1).all()
+            else:
+                assert sorted(p[0] for p in pieces) == list(range(len(pieces))) and len(pieces) <= max_chunks
+                assert (token_chunks[tb:tb + count] == len(pieces)).all()
