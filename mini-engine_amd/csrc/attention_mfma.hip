@@ -98,7 +98,7 @@ __device__ __forceinline__ void load_tile(KvTile<D>& t, const bf16_t* __restrict
 template <int D, int NB>
 __device__ __forceinline__ void compute_tile(const KvTile<D>& t, int key0, int lo, const int (&qpos)[NB],
                                              bool need_mask, const Frag8 (&qf)[NB][D / 32], float scale_log2,
-                                             float (&m)[NB], float (&lsum)[NB], float4_t (&acc)[NB][D / 16]) {
+                                             float (&m)[NB], float (&lsum)[NB], float4_t (&acc)[NB][D / 16], int keep_first = 0) {
   const int lane = threadIdx.x & (ME_WAVE - 1);
   const int g = lane >> 4;
   short4_t pf[NB];
@@ -116,7 +116,7 @@ __device__ __forceinline__ void compute_tile(const KvTile<D>& t, int key0, int l
       sv[i] = s[i] * scale_log2;
       if (need_mask) {
         const int key = key0 + g * 4 + i;
-        if (key < lo || key > qpos[nb]) sv[i] = -INFINITY;
+        if ((key < lo && key >= keep_first) || key > qpos[nb]) sv[i] = -INFINITY;
       }
     }
     float tmax = column_max(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])));
@@ -167,6 +167,9 @@ struct DecodeFusedArgs {
   int write_kv;             // 0: a layer that reads another layer's cache
   bf16_t* k_cache_w;
   bf16_t* v_cache_w;
+  // (for every launch, fused or not) with a window: the first keys of an item that stay visible behind it. Their tiles
+  // come before the window's in the order in which an item's tiles are dealt to the splits.
+  int keep_first = 0;
 };
 
 // Tiles of a split from which on a wave fetches one tile at a time, whatever DEPTH says: with five tiles and more of its own
@@ -221,7 +224,13 @@ __device__ __forceinline__ void attention_decode_body(
   }
   const int lo = window > 0 ? max(ctx - window, 0) : 0;
   const int lo16 = (lo / 16) * 16;
-  int tiles_per_split = ((ctx - lo16 + 15) / 16 + splits - 1) / splits;
+  // Kept first keys that the window has left behind: their tiles (keys 0 .. kept16 - 1) stand before the window's, at the
+  // places vlo .. lo16 - 1 of the run of tiles that is dealt to the splits; `key_at` gives a place's key.
+  const int keep_first = fa.keep_first;
+  const int kept16 = keep_first > 0 && lo16 > 0 ? min((keep_first + 15) / 16 * 16, lo16) : 0;
+  const int vlo = lo16 - kept16;
+  auto key_at = [&](int place) { return place < lo16 ? place - vlo : place; };
+  int tiles_per_split = ((ctx - vlo + 15) / 16 + splits - 1) / splits;
   // With 16 splits and more per item, runs of 16, 32, 48 or 64 tiles (the waves of an item then start at keys a multiple of 256
   // apart and walk them in step) measured slower than runs one tile longer with a split less at work, on the same GPU in turns:
   // batch 8 at a context of 8,192 2.78 -> 2.44 ms a step, batch 4 at 8,192 1.98 -> 1.76, batch 8 at 4,096 1.83 -> 1.78 in a
@@ -232,7 +241,7 @@ __device__ __forceinline__ void attention_decode_body(
   // the longer runs cost what they are longer (batch 16 at 4,096, 8 splits of 32 tiles: 2.374 -> 2.430), so those keep
   // theirs, and so do blocks that add up their own waves' splits.
   if (block_waves == 1 && splits >= 16 && tiles_per_split % 16 == 0 && tiles_per_split <= 64) ++tiles_per_split;
-  const int begin = lo16 + split * tiles_per_split * 16;
+  const int begin = vlo + split * tiles_per_split * 16;
   const int end = min(begin + tiles_per_split * 16, ctx);
 
   float m[1] = {-INFINITY}, lsum[1] = {0.f};
@@ -244,7 +253,7 @@ __device__ __forceinline__ void attention_decode_body(
     // the first tile is requested before the query is prepared, unless it holds the slot that this
     // block is about to write
     const bool early = !FUSED || begin + 16 < ctx;
-    if (early) fetch(t[0], begin);
+    if (early) fetch(t[0], key_at(begin));
     Frag8 qf[1][D / 32];
     if (FUSED) {
       constexpr int HC = D / 64;  // chunks per half head
@@ -341,7 +350,7 @@ __device__ __forceinline__ void attention_decode_body(
       }
     }
     const int qpos[1] = {ctx - 1};
-    if (!early) fetch(t[0], begin);
+    if (!early) fetch(t[0], key_at(begin));
     // DEPTH tiles in flight per wave: tile i + DEPTH - 1 is requested before the products of tile i. Short
     // splits (few waves, each waiting on memory) want two (four measured no better); with long splits the
     // chip is full of waves and fewer registers, one more wave per SIMD, serve better. A tile past `end` is a valid page that
@@ -349,20 +358,20 @@ __device__ __forceinline__ void attention_decode_body(
     if (DEPTH > 1 && tiles_per_split > LONG_RUN) {
       // a long run of this wave's own (the chip is full of such waves): one tile at a time streams best
       for (int k = begin; k < end; k += 16) {
-        if (k > begin) fetch(t[0], k);
-        compute_tile<D, 1>(t[0], k, lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc);
+        if (k > begin) fetch(t[0], key_at(k));
+        compute_tile<D, 1>(t[0], key_at(k), lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc, keep_first);
       }
     } else {
 #pragma unroll
-      for (int j = 1; j < DEPTH - 1; ++j) fetch(t[j], begin + 16 * j);
+      for (int j = 1; j < DEPTH - 1; ++j) fetch(t[j], key_at(begin + 16 * j));
       for (int key0 = begin; key0 < end; key0 += 16 * DEPTH) {
 #pragma unroll
         for (int j = 0; j < DEPTH; ++j) {
           const int k = key0 + 16 * j;
-          if (DEPTH > 1) fetch(t[(j + DEPTH - 1) % DEPTH], k + 16 * (DEPTH - 1));
-          else if (k > begin) fetch(t[0], k);
+          if (DEPTH > 1) fetch(t[(j + DEPTH - 1) % DEPTH], key_at(k + 16 * (DEPTH - 1)));
+          else if (k > begin) fetch(t[0], key_at(k));
           if (j == 0 || k < end)
-            compute_tile<D, 1>(t[j], k, lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc);
+            compute_tile<D, 1>(t[j], key_at(k), lo, qpos, k < lo || k + 16 > ctx, qf, scale_log2, m, lsum, acc, keep_first);
         }
       }
     }
@@ -543,7 +552,9 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
                           int width, float* part_o, float* part_ml, int items, int nh, int nkv, int bs, int window,
                           float scale_log2, int depth, int num_splits, int block_waves, bf16_t* out,
                           const DecodeFusedArgs* fused, const int* live_items, int waves_wanted, int streamed,
-                          const int* step_flags, hipStream_t stream) {
+                          const int* step_flags, int keep_first, hipStream_t stream) {
+  DecodeFusedArgs unfused{};
+  unfused.keep_first = keep_first;
   const int chunks = (nh / nkv + 15) / 16;
   dim3 grid(items, nkv * chunks, num_splits / block_waves);  // num_splits is a multiple of block_waves
   const int heads_most = nh / nkv < 16 ? nh / nkv : 16;
@@ -571,9 +582,9 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
     }
   }
   if (depth == 2)
-    ME_DECODE_LAUNCH(false, 2, DecodeFusedArgs{});
+    ME_DECODE_LAUNCH(false, 2, unfused);
   else
-    ME_DECODE_LAUNCH(false, 1, DecodeFusedArgs{});
+    ME_DECODE_LAUNCH(false, 1, unfused);
 #undef ME_DECODE_LAUNCH_AS
 #undef ME_DECODE_LAUNCH
 }
@@ -635,7 +646,19 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
                          int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
-                         int waves_wanted, const int* step_flags, hipStream_t stream);
+                         int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first = 0);
+
+// As me_attention_decode_bf16, with the first `keep_first` keys of every item visible behind the window.
+extern "C" int me_attention_decode_bf16_kept(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
+                                             const int* block_table, int table_width, void* out, float* part_o,
+                                             float* part_ml, int items, int nh, int nkv, int d, int bs, int window,
+                                             int keep_first, float scale, int split_keys, int num_splits, int max_ctx,
+                                             const int* live_items, int full_splits, int waves_wanted,
+                                             const int* step_flags, hipStream_t stream) {
+  return decode_common(q, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
+                       bs, window, scale, split_keys, num_splits, max_ctx, nullptr, live_items, full_splits, waves_wanted,
+                       step_flags, stream, keep_first);
+}
 
 extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
                                         const int* block_table, int table_width, void* out, float* part_o,
@@ -685,8 +708,10 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
                          int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
-                         int waves_wanted, const int* step_flags, hipStream_t stream) {
+                         int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first) {
   if (items <= 0) return 0;
+  if (keep_first < 0 || (keep_first > 0 && (window <= 0 || fused)))
+    return me_fail("me_attention_decode_bf16: keep_first=%d needs a window and the unfused form", keep_first);
   if (!me_attention_mfma_supported(d, bs))
     return me_fail("me_attention_decode_bf16: head_dim=%d / block_size=%d not supported by the matrix-core kernels", d, bs);
   if (nh <= 0 || nkv <= 0 || nh % nkv) return me_fail("me_attention_decode_bf16: nh=%d nkv=%d", nh, nkv);
@@ -724,7 +749,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   case DD:                                                                                                      \
     launch_decode<DD>(qq, kc, vc, item_ctx, block_table, table_width, part_o, part_ml, items, nh, nkv, bs, window, sl, \
                       depth, num_splits, block_waves, (bf16_t*)out, fused, live_items, waves_wanted, streamed, step_flags, \
-                      stream);                                                                                  \
+                      keep_first, stream);                                                                      \
     break;
   switch (d) {
     ME_DECODE_CASE(32)

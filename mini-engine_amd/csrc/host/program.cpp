@@ -438,6 +438,19 @@ class Run {
       void* q = arena_.take((size_t)t_ * nh * d * elem_);
       ok(me_qkv_rotate_scatter(qkv, q_w, k_w, rope, rd, pairing, v_table, v_pairing, idx(s_.lay.positions), idx(s_.lay.token_item),
                                table, width, q, kc, vc, t_, nh, nkv, d, dv, bs, eps, dtype_, stream_));
+      if (s_.decode_only && attention_takes_tiled_prefill(op, dtype_)) {
+        // one new token per item: the split-context kernel, which deals the kept first keys' tiles to its splits before
+        // the window's; a second kernel (or the blocks themselves) adds up the splits
+        if ((long long)width * bs < s_.max_ctx) throw Error(kBadValue, "the block table cannot hold the step's longest context");
+        const SplitPlan sp = split_plan(items, nkv * ((group + 15) / 16), s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
+        float* part_o = (float*)arena_.take((size_t)items * nh * sp.num_splits * d * 4);
+        float* part_ml = (float*)arena_.take((size_t)items * nh * sp.num_splits * 2 * 4);
+        ok(me_attention_decode_bf16_kept(q, kc, vc, idx(s_.lay.item_ctx), table, width, out, part_o, part_ml, items, nh, nkv, d, bs,
+                                         window, keep_first, scale, sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits,
+                                         kDecodeWaves, idx(s_.lay.live_items) + 1, stream_));
+        if (v_table) ok(me_unturn_rows(out, v_table, v_pairing, idx(s_.lay.positions), t_, nh, dv, dtype_, stream_));
+        return;
+      }
       if (!s_.decode_only && attention_takes_tiled_prefill(op, dtype_)) {
         // prompts and portions in bfloat16 with keys and values of one size the matrix cores take: the tiled kernel, whose
         // work list has an entry of its own for the kept first keys; the outputs are turned back by a pass of their own
@@ -671,6 +684,16 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
       need = (size_t)me_decay_state_workspace(tokens, items, (int)op.i[0], (int)op.i[1], (int)op.i[2]) + pad;
     if (op.kind == kOpAttention && !attention_is_plain(op)) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
+      if (attention_takes_tiled_prefill(op, dtype_)) {  // the splits' partial results of a decode step
+        const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2];
+        size_t most = 0;
+        for (int64_t b = 1; b <= items; ++b) {
+          int keys, splits;
+          decode_splits((int)std::max<int64_t>(1, (b + 1) / 2), nkv * ((nh / nkv + 15) / 16), (int)max_ctx, keys, splits);
+          most = std::max(most, (size_t)b * splits);
+        }
+        need += most * nh * (d + 2) * 4 + 2 * pad;
+      }
       if (attention_takes_tiled_prefill(op, dtype_) && tokens > items)  // partial results of cut tiles: the work list's bound,
         need += (size_t)(256ll << 20) + (size_t)(256ll << 20) * 2 / op.i[2] +  // and one chunk more for the kept first keys
                 (size_t)tokens * op.i[0] * (op.i[2] + 2) * 4 * 2 + 2 * pad;

@@ -919,13 +919,14 @@ def attention_decode_leaves_parts(items: int, num_heads: int, num_kv_heads: int,
 
 def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: float, window: int, max_ctx: int,
                           out: torch.Tensor | None = None, live=None, step_flags: torch.Tensor | None = None,
-                          leave_parts: bool = False):
+                          leave_parts: bool = False, keep_first: int = 0):
     """Attention of one new token per item over its cached keys: q [items, nh, d] bfloat16,
     item_ctx int32 [items] (keys per item, the new one included, each <= max_ctx). ``live``: see
     :func:`_decode_split_plan`. ``step_flags``: None, or a device int32 whose bit 0 says that the items share
     pages (a large launch then loads keys and values with ordinary loads instead of non-temporal ones).
     ``leave_parts``: the splits are not added up; the result is ``(part_o, part_ml, num_splits)`` for
-    :func:`attention_out_product_bf16` (only where :func:`attention_decode_leaves_parts` says so)."""
+    :func:`attention_out_product_bf16` (only where :func:`attention_decode_leaves_parts` says so).
+    ``keep_first``: with a window, the first keys of every item that stay visible behind it."""
     _want(q, "q", torch.bfloat16, (None, None, None))
     items, nh, d = q.shape
     nkv, bs = k_cache.shape[1], k_cache.shape[2]
@@ -944,9 +945,9 @@ def attention_decode_bf16(q, k_cache, v_cache, item_ctx, block_table, scale: flo
         if out is None:
             out = torch.empty((items, nh * d), dtype=torch.bfloat16, device=q.device)
         _want(out, "out", torch.bfloat16, (items, nh * d))
-    check(lib().me_attention_decode_bf16(
+    check(lib().me_attention_decode_bf16_kept(
         _p(q), _p(k_cache), _p(v_cache), _p(item_ctx), _p(block_table), _i(block_table.shape[1]), _p(out),
-        _p(part_o), _p(part_ml), _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _f(scale), _i(split_keys),
+        _p(part_o), _p(part_ml), _i(items), _i(nh), _i(nkv), _i(d), _i(bs), _i(window), _i(keep_first), _f(scale), _i(split_keys),
         _i(num_splits), _i(max_ctx), _p(live_count), _i(full_splits), _i(DECODE_WAVES), _p(step_flags), _stream()))
     return (part_o, part_ml, num_splits) if leave_parts else out
 

@@ -126,8 +126,16 @@ class Attention(Mixer):
             v_pairing = 0 if self.value_position is None else self.value_position.pairing_code
             q = K.qkv_rotate_scatter(proj, self.q_norm_w, self.k_norm_w, rope, self.pairing, vt, v_pairing, batch.positions,
                                      batch.token_item, table, b.k_cache, b.v_cache, self.nh, self.nkv, self.d, self.dv, eps)
-            if (self.dtype is torch.bfloat16 and not batch.decode_only and self.dv == self.d
-                    and K.attention_mfma_supported(self.d, b.block_size, self.nh // self.nkv)):
+            tiled = (self.dtype is torch.bfloat16 and self.dv == self.d
+                     and K.attention_mfma_supported(self.d, b.block_size, self.nh // self.nkv))
+            if tiled and batch.decode_only:  # one new token per item: the split-context matrix-core kernel
+                out = K.attention_decode_bf16(q, b.k_cache, b.v_cache, batch.item_ctx, table, float(s.scale), int(s.window),
+                                              batch.max_ctx, live=(batch.live_items, batch.least_live),
+                                              keep_first=self.keep_first)
+                if vt is not None:
+                    K.unturn_rows(out, vt, v_pairing, batch.positions, self.nh)
+                return K.linear(out, self.w_o, as_delta=True)
+            if tiled:
                 # prompts and portions: the tiled matrix-core kernel, then the outputs turned back in a pass of their own
                 key = ("prefill_plan", self.nh, self.nkv, self.d, int(s.window), self.keep_first)
                 plan = batch.derived.get(key)

@@ -192,6 +192,19 @@ def test_tiled_prompt_attention_sees_the_kept_first_keys(nh, nkv, d, rd, pairing
         # the kernel that takes every size, on the same pages: the two differ by the rounding of the weights alone
         same = K.attention_general(q, k_cache, v_cache, pos, item, table, scale, size, keep_first=keep, unturn=vt, un_pairing=code)
         assert rel_err(out, same) < 2e-2
+    # one new token per item over the same pages: the split-context kernel deals the kept keys' tiles to its splits too
+    for ends in ((330, 205), (329, 201), (215, 78)):
+        pos = torch.tensor([e - 1 for e in ends], dtype=torch.int32).cuda()
+        item = torch.tensor([0, 1], dtype=torch.int32).cuda()
+        rows = torch.stack([seqs[i][e - 1] for i, e in enumerate(ends)]).cuda().contiguous()
+        q = K.qkv_rotate_scatter(rows, None, None, rope, code, vt, code, pos, item, table, k_cache, v_cache, nh, nkv, d, d, eps)
+        ctx = torch.tensor(list(ends), dtype=torch.int32).cuda()
+        out = K.attention_decode_bf16(q, k_cache, v_cache, ctx, table, scale, size, table.shape[1] * bs, keep_first=keep)
+        K.unturn_rows(out, vt, code, pos, nh)
+        same = K.attention_general(q, k_cache, v_cache, pos, item, table, scale, size, keep_first=keep, unturn=vt, un_pairing=code)
+        assert rel_err(out, same) < 2e-2
+        for i, e in enumerate(ends):
+            assert rel_err(out[i : i + 1], wants[i][e - 1 : e]) < 8e-2
     for i in range(2):
         # (scores this loud feel the rounding of the turned q and k: both kernels are up to 6% of a row's largest value off)
         assert rel_err(torch.cat(got[i]), wants[i]) < 8e-2
