@@ -78,9 +78,14 @@ __global__ __launch_bounds__(256) void decay_state_prepare_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------- scan
-// A wave owns 16 columns of the state: lane = rg * 16 + column, rg = 0..3 the quarter of the rows (RPL rows a lane,
-// 4 * RPL >= d; q32 and k32 rows are padded to 4 * RPL with zeros). The next token's q, k and v are requested before
-// the current token's arithmetic. Three forms:
+// A wave owns 16 * CPL columns of the state: lane = rg * 16 + c, rg = 0..3 the quarter of the rows (RPL rows a lane,
+// 4 * RPL >= d; q32 and k32 rows are padded to 4 * RPL with zeros), c the lane's CPL neighbouring columns. The 16 lanes
+// of a quarter read the same rows of k (and q): fetched from memory by every lane for itself, those reads kept the load
+// path busy for longer than the arithmetic takes, so the chunked forms stage a chunk's rows in LDS once per block
+// (a 2,048-token prompt, 16 heads of 128 x 128: the outputs 171 -> 114 us a layer), and the sums' form, which holds no
+// q, gives a lane two columns (96 -> 57 us; the outputs' form with two columns a lane was slower, 193 us without the
+// staging). A sum's order does not depend on any of this. The next token's q, k and v are requested before the current
+// token's arithmetic. Three forms:
 //
 //   DS_WHOLE   grid (item, head, 64 columns): the item's new tokens in order, from the state in its slot, which is left
 //              updated. The decay is applied as two floats. Decode steps and short portions.
@@ -112,17 +117,23 @@ __device__ __forceinline__ bool ds_chunk_tokens(const int* __restrict__ item_sta
   return false;
 }
 
-template <int RPL, int MODE>
+template <int RPL, int MODE, int CPL>
 __global__ __launch_bounds__(256) void decay_state_scan_kernel(
     const float* __restrict__ q32, const float* __restrict__ k32, const float* __restrict__ v32, float* __restrict__ o32,
     float* __restrict__ state, float* __restrict__ chunks, const float* __restrict__ decay, const int* __restrict__ item_start,
     const int* __restrict__ state_slots, int items, int heads, int d, int dv) {
   constexpr int DP = 4 * RPL;
+  constexpr int QUARTER = RPL + 4, LROW = 4 * QUARTER;  // a row of k or q in LDS: its four quarters 16 bytes apart from a
+                                                        // multiple of 128, so that the four addresses of a read hit other banks
+  extern __shared__ __attribute__((aligned(16))) float ds_lds[];  // the chunked forms: [64][LROW] of k, then of q
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int head = blockIdx.y;
-  const int col = (blockIdx.z * 4 + wave) * 16 + (lane & 15), rg = lane >> 4;
-  if ((blockIdx.z * 4 + wave) * 16 >= dv) return;  // (whole waves: no block-wide barrier below)
-  const bool has_col = col < dv;
+  const int col = ((blockIdx.z * 4 + wave) * 16 + (lane & 15)) * CPL, rg = lane >> 4;  // the first of this lane's columns
+  const bool idle = (blockIdx.z * 4 + wave) * 16 * CPL >= dv;  // a wave beyond the last column
+  if (MODE == DS_WHOLE && idle) return;
+  bool has_col[CPL];
+#pragma unroll
+  for (int c = 0; c < CPL; ++c) has_col[c] = col + c < dv;
   int item = blockIdx.x, t0, t1;
   if (MODE == DS_WHOLE) {
     t0 = item_start[item], t1 = item_start[item + 1];
@@ -130,28 +141,47 @@ __global__ __launch_bounds__(256) void decay_state_scan_kernel(
     return;
   }
   const int slot = state_slots[item];
-  if (slot < 0 || t1 <= t0) return;
+  if (slot < 0 || t1 <= t0) return;  // (the same for every thread of the block)
+  if (MODE != DS_WHOLE) {
+    // The chunk's rows of k (and q) go to LDS once for the block's four waves: fetched by every lane for itself they
+    // keep the load path busy for longer than the arithmetic takes (the 16 lanes of a quarter read the same 16 bytes).
+    const int pieces = (t1 - t0) * (DP / 4);
+    for (int idx = threadIdx.x; idx < pieces; idx += blockDim.x) {
+      const int tt = idx / (DP / 4), p = idx % (DP / 4);
+      const size_t row = ((size_t)(t0 + tt) * heads + head) * DP;
+      const int at = tt * LROW + (p / (RPL / 4)) * QUARTER + (p % (RPL / 4)) * 4;
+      *reinterpret_cast<float4*>(ds_lds + at) = reinterpret_cast<const float4*>(k32 + row)[p];
+      if (MODE == DS_OUTPUTS) *reinterpret_cast<float4*>(ds_lds + DS_CHUNK * LROW + at) = reinterpret_cast<const float4*>(q32 + row)[p];
+    }
+    __syncthreads();
+    if (idle) return;
+  }
   const float lam = decay[head], lam_lo = MODE == DS_WHOLE ? decay[heads + head] : 0.f;
   float* srow = MODE == DS_WHOLE ? state + (((size_t)slot * heads + head) * d) * dv
                                  : chunks + (((size_t)blockIdx.x * heads + head) * d) * dv;  // [d, dv]
-  float S[RPL];
+  float S[CPL][RPL];
 #pragma unroll
-  for (int r = 0; r < RPL; ++r) {
-    const int i = rg * RPL + r;
-    S[r] = MODE != DS_SUMS && has_col && i < d ? srow[(size_t)i * dv + col] : 0.f;
-  }
+  for (int c = 0; c < CPL; ++c)
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+      const int i = rg * RPL + r;
+      S[c][r] = MODE != DS_SUMS && has_col[c] && i < d ? srow[(size_t)i * dv + col + c] : 0.f;
+    }
   float4 qn[RPL / 4], kn[RPL / 4];
-  float vn;
+  float vn[CPL];
   auto fetch = [&](int t) {
-    const float4* kp = reinterpret_cast<const float4*>(k32 + ((size_t)t * heads + head) * DP + rg * RPL);
+    const float4* kp = MODE == DS_WHOLE ? reinterpret_cast<const float4*>(k32 + ((size_t)t * heads + head) * DP + rg * RPL)
+                                        : reinterpret_cast<const float4*>(ds_lds + (t - t0) * LROW + rg * QUARTER);
 #pragma unroll
     for (int r = 0; r < RPL / 4; ++r) kn[r] = kp[r];
     if (MODE != DS_SUMS) {
-      const float4* qp = reinterpret_cast<const float4*>(q32 + ((size_t)t * heads + head) * DP + rg * RPL);
+      const float4* qp = MODE == DS_WHOLE ? reinterpret_cast<const float4*>(q32 + ((size_t)t * heads + head) * DP + rg * RPL)
+                                          : reinterpret_cast<const float4*>(ds_lds + DS_CHUNK * LROW + (t - t0) * LROW + rg * QUARTER);
 #pragma unroll
       for (int r = 0; r < RPL / 4; ++r) qn[r] = qp[r];
     }
-    vn = has_col ? v32[((size_t)t * heads + head) * dv + col] : 0.f;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) vn[c] = has_col[c] ? v32[((size_t)t * heads + head) * dv + col + c] : 0.f;
   };
   fetch(t0);
   for (int t = t0; t < t1; ++t) {
@@ -162,37 +192,50 @@ __global__ __launch_bounds__(256) void decay_state_scan_kernel(
 #pragma unroll
       for (int r = 0; r < RPL / 4; ++r) qc[r] = qn[r];
     }
-    const float vc = vn;
+    float vc[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) vc[c] = vn[c];
     if (t + 1 < t1) fetch(t + 1);
-    float o = 0.f;
+    float o[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) o[c] = 0.f;
 #pragma unroll
     for (int r = 0; r < RPL / 4; ++r) {
       const float kk[4] = {kc[r].x, kc[r].y, kc[r].z, kc[r].w};
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float s = S[4 * r + u];
-        float sn = fmaf(lam, s, kk[u] * vc);
-        if (MODE == DS_WHOLE) sn = fmaf(lam_lo, s, sn);
-        S[4 * r + u] = sn;
-      }
+      for (int c = 0; c < CPL; ++c)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const float s = S[c][4 * r + u];
+          float sn = fmaf(lam, s, kk[u] * vc[c]);
+          if (MODE == DS_WHOLE) sn = fmaf(lam_lo, s, sn);
+          S[c][4 * r + u] = sn;
+        }
       if (MODE != DS_SUMS) {
         const float qq[4] = {qc[r].x, qc[r].y, qc[r].z, qc[r].w};
 #pragma unroll
-        for (int u = 0; u < 4; ++u) o = fmaf(S[4 * r + u], qq[u], o);
+        for (int c = 0; c < CPL; ++c)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) o[c] = fmaf(S[c][4 * r + u], qq[u], o[c]);
       }
     }
     if (MODE != DS_SUMS) {
-      o += __shfl_xor(o, 16, ME_WAVE);
-      o += __shfl_xor(o, 32, ME_WAVE);
-      if (rg == 0 && has_col) o32[((size_t)t * heads + head) * dv + col] = o;
+#pragma unroll
+      for (int c = 0; c < CPL; ++c) {
+        o[c] += __shfl_xor(o[c], 16, ME_WAVE);
+        o[c] += __shfl_xor(o[c], 32, ME_WAVE);
+        if (rg == 0 && has_col[c]) o32[((size_t)t * heads + head) * dv + col + c] = o[c];
+      }
     }
   }
   if (MODE == DS_OUTPUTS) return;
 #pragma unroll
-  for (int r = 0; r < RPL; ++r) {
-    const int i = rg * RPL + r;
-    if (has_col && i < d) srow[(size_t)i * dv + col] = S[r];
-  }
+  for (int c = 0; c < CPL; ++c)
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+      const int i = rg * RPL + r;
+      if (has_col[c] && i < d) srow[(size_t)i * dv + col + c] = S[c][r];
+    }
 }
 
 // The states at the chunks' starts, in place of the chunks' sums: per item, head and element of the state,
@@ -262,6 +305,24 @@ __global__ __launch_bounds__(256) void decay_state_finish_kernel(const float* __
   }
 }
 
+// One instance of the scan: the chunked forms stage k (and q) in LDS, more than a launch may take without asking.
+template <int RPL, int MODE, int CPL>
+static int launch_scan(dim3 grid, hipStream_t stream, const float* q32, const float* k32, const float* v32, float* o32, float* state,
+                       float* chunks, const float* decay, const int* item_start, const int* state_slots, int items, int heads,
+                       int d, int dv) {
+  const size_t lds = MODE == DS_WHOLE ? 0 : (size_t)(MODE == DS_OUTPUTS ? 2 : 1) * DS_CHUNK * 4 * (RPL + 4) * sizeof(float);
+  static bool configured = false;
+  if (lds > 48 * 1024 && !configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&decay_state_scan_kernel<RPL, MODE, CPL>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return me_fail("me_decay_state: %zu bytes of block memory are refused", lds);
+    configured = true;
+  }
+  decay_state_scan_kernel<RPL, MODE, CPL><<<grid, 256, lds, stream>>>(q32, k32, v32, o32, state, chunks, decay, item_start,
+                                                                      state_slots, items, heads, d, dv);
+  return 0;
+}
+
 // --------------------------------------------------------------------------------------------- entry points
 extern "C" int me_decay_state_padded_dim(int d) {  // the row length of the prepared q and k
   return d <= 32 ? 32 : d <= 64 ? 64 : d <= 128 ? 128 : 256;
@@ -305,12 +366,23 @@ extern "C" int me_decay_state(const void* proj, const float* rope_table, int rd,
   // step side by side. Else every item in order, a block per item, head and 64 columns.
   const bool by_chunks = longest_item > 2 * DS_CHUNK;
   const int num_chunks = num_tokens / DS_CHUNK + items;  // an upper bound: blocks beyond the last chunk leave at once
+  // two columns a lane where the rows a lane holds leave the registers for it and the heads are wide enough to fill the waves
+  const int cpl = by_chunks && dp <= 128 && dv >= 32 ? 2 : 1;
   const dim3 scan_grid(by_chunks ? num_chunks : items, heads, (dv + 63) / 64);
+  const dim3 scan_grid2(scan_grid.x, heads, (dv + 127) / 128);  // two columns a lane
   if (scan_grid.z > 65535 || (long long)d * dv > (1ll << 24)) return me_fail("me_decay_state: value heads of %d elements", dv);
   const dim3 starts_grid((d * dv + 255) / 256, heads, items);
 #define DS_SCAN_MODE(RPL, MODE)                                                                                              \
-  decay_state_scan_kernel<RPL, MODE><<<scan_grid, 256, 0, stream>>>(q32, k32, v32, o32, state, chunk_states, decay, item_start, \
-                                                                    state_slots, items, heads, d, dv)
+  do {                                                                                                                       \
+    int failed;                                                                                                              \
+    if (cpl == 2 && RPL <= 32 && MODE == DS_SUMS)                                                                            \
+      failed = launch_scan<(RPL <= 32 ? RPL : 8), MODE, 2>(scan_grid2, stream, q32, k32, v32, o32, state, chunk_states, decay,  \
+                                                           item_start, state_slots, items, heads, d, dv);                     \
+    else                                                                                                                     \
+      failed = launch_scan<RPL, MODE, 1>(scan_grid, stream, q32, k32, v32, o32, state, chunk_states, decay, item_start,         \
+                                         state_slots, items, heads, d, dv);                                                   \
+    if (failed) return failed;                                                                                               \
+  } while (0)
 #define DS_SCAN(RPL)                                                                                                         \
   do {                                                                                                                       \
     if (by_chunks) {                                                                                                         \

@@ -965,7 +965,7 @@ extern "C" int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const fl
   if (nh <= 0 || nkv <= 0 || bs <= 0 || table_width <= 0)
     return me_fail("me_qkv_rotate_scatter: nh=%d nkv=%d block_size=%d table_width=%d", nh, nkv, bs, table_width);
   const int heads_total = nh + 2 * nkv;
-  const int hpb = num_tokens >= 512 ? heads_total : 4;
+  const int hpb = num_tokens >= 512 ? 8 : 4;  // heads a block of four waves takes, a wave a head at a time
   dim3 grid(num_tokens, (heads_total + hpb - 1) / hpb);
   if (grid.y > 65535) return me_fail("me_qkv_rotate_scatter: too many heads");
   if (dtype == ME_F32)
