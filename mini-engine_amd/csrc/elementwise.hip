@@ -744,14 +744,16 @@ extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const 
 //   the row is cut into `groups` equal consecutive parts, each divided by its own sqrt(mean(part^2) + eps);
 //   h[r] = that, times w.
 // One block per row, a wave per group at a time: a group's sum of squares is added up in an order that its length
-// alone fixes. groups == 1 and delta_scale == 1 is the norm of the kernels above.
+// alone fixes. groups == 1 and delta_scale == 1 is the norm of the kernels above. A second delta (`delta2` or `parts2`,
+// the result of a part that ran beside the first on the same normed input) is added with the same scale.
 #define ME_MAX_NORM_GROUPS 64
 
 template <typename T>
 __global__ void add_group_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ parts,
-                                         int num_parts, size_t part_stride, float delta_scale, const float* __restrict__ w,
-                                         T* __restrict__ h, const int* __restrict__ rows, int dim, int groups, float eps,
-                                         int write_x) {
+                                         int num_parts, size_t part_stride, const T* __restrict__ delta2,
+                                         const float* __restrict__ parts2, int num_parts2, size_t part_stride2, float delta_scale,
+                                         const float* __restrict__ w, T* __restrict__ h, const int* __restrict__ rows, int dim,
+                                         int groups, float eps, int write_x) {
   __shared__ float inv[ME_MAX_NORM_GROUPS];
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1), waves = blockDim.x / ME_WAVE;
   const int r = blockIdx.x;
@@ -759,17 +761,31 @@ __global__ void add_group_rmsnorm_kernel(float* __restrict__ x, const T* __restr
   float* xr = x + (size_t)src * dim;
   const T* dr = delta ? delta + (size_t)src * dim : nullptr;
   const float* pr = parts ? parts + (size_t)src * dim : nullptr;
-  const bool adds = dr || pr;
+  const T* dr2 = delta2 ? delta2 + (size_t)src * dim : nullptr;
+  const float* pr2 = parts2 ? parts2 + (size_t)src * dim : nullptr;
+  const bool adds = dr || pr || dr2 || pr2;
   const int gs = dim / groups;
+  // partial sums in the order of their runs, eight requested at a time (a run beyond the last reads the last one again
+  // and counts for nothing): one trip to memory for eight instead of one for each
+  auto sum_parts = [&](const float* at, int n, size_t stride) {
+    float q = 0.f;
+    for (int p0 = 0; p0 < n; p0 += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = at[(size_t)min(p0 + u, n - 1) * stride];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) q += p0 + u < n ? v[u] : 0.f;
+    }
+    return q;
+  };
   auto sum_at = [&](int i) {
+    const float x0 = xr[i];
     float d = 0.f;
     if (dr) d = to_float(dr[i]);
-    if (pr) {
-      float q = pr[i];
-      for (int p = 1; p < num_parts; ++p) q += pr[p * part_stride + i];
-      d += q;
-    }
-    return adds ? fmaf(delta_scale, d, xr[i]) : xr[i];
+    if (pr) d += sum_parts(pr + i, num_parts, part_stride);
+    if (dr2) d += to_float(dr2[i]);
+    if (pr2) d += sum_parts(pr2 + i, num_parts2, part_stride2);
+    return adds ? fmaf(delta_scale, d, x0) : x0;
   };
   for (int g = wave; g < groups; g += waves) {
     float ss = 0.f;
@@ -789,23 +805,32 @@ __global__ void add_group_rmsnorm_kernel(float* __restrict__ x, const T* __restr
   }
 }
 
-extern "C" int me_add_group_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride,
-                                    float delta_scale, const float* w, void* h, const int* rows, int num_rows, int dim,
-                                    int groups, float eps, int write_x, int dtype, hipStream_t stream) {
+extern "C" int me_add_group_rmsnorm2(void* x, const void* delta, const float* parts, int num_parts, long long part_stride,
+                                     const void* delta2, const float* parts2, int num_parts2, long long part_stride2,
+                                     float delta_scale, const float* w, void* h, const int* rows, int num_rows, int dim,
+                                     int groups, float eps, int write_x, int dtype, hipStream_t stream) {
   if (num_rows <= 0) return 0;
   if (dim <= 0 || groups < 1 || groups > ME_MAX_NORM_GROUPS || dim % groups)
     return me_fail("me_add_group_rmsnorm: dim=%d in %d groups (1..%d equal parts)", dim, groups, ME_MAX_NORM_GROUPS);
   if (parts && (num_parts < 1 || part_stride < (long long)dim)) return me_fail("me_add_group_rmsnorm: %d partial sums", num_parts);
+  if (parts2 && (num_parts2 < 1 || part_stride2 < (long long)dim)) return me_fail("me_add_group_rmsnorm: %d partial sums", num_parts2);
   const int threads = dim >= 1024 ? 256 : (dim >= 256 ? 128 : 64);
   if (dtype == ME_F32)
-    add_group_rmsnorm_kernel<float><<<num_rows, threads, 0, stream>>>((float*)x, (const float*)delta, parts, num_parts,
-                                                                      (size_t)part_stride, delta_scale, w, (float*)h, rows, dim,
-                                                                      groups, eps, write_x);
+    add_group_rmsnorm_kernel<float><<<num_rows, threads, 0, stream>>>(
+        (float*)x, (const float*)delta, parts, num_parts, (size_t)part_stride, (const float*)delta2, parts2, num_parts2,
+        (size_t)part_stride2, delta_scale, w, (float*)h, rows, dim, groups, eps, write_x);
   else
-    add_group_rmsnorm_kernel<bf16_t><<<num_rows, threads, 0, stream>>>((float*)x, (const bf16_t*)delta, parts, num_parts,
-                                                                       (size_t)part_stride, delta_scale, w, (bf16_t*)h, rows,
-                                                                       dim, groups, eps, write_x);
+    add_group_rmsnorm_kernel<bf16_t><<<num_rows, threads, 0, stream>>>(
+        (float*)x, (const bf16_t*)delta, parts, num_parts, (size_t)part_stride, (const bf16_t*)delta2, parts2, num_parts2,
+        (size_t)part_stride2, delta_scale, w, (bf16_t*)h, rows, dim, groups, eps, write_x);
   return me_check_launch("me_add_group_rmsnorm");
+}
+
+extern "C" int me_add_group_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride,
+                                    float delta_scale, const float* w, void* h, const int* rows, int num_rows, int dim,
+                                    int groups, float eps, int write_x, int dtype, hipStream_t stream) {
+  return me_add_group_rmsnorm2(x, delta, parts, num_parts, part_stride, nullptr, nullptr, 0, 0, delta_scale, w, h, rows, num_rows,
+                               dim, groups, eps, write_x, dtype, stream);
 }
 
 // x += scale * (delta + the partial sums, in the order of the runs): the residual add of a block that multiplies

@@ -218,6 +218,14 @@ class Run {
       case kOpDecayState:
         decay_state(op);
         break;
+      case kOpHold:
+        if (held_.any()) throw Error(kBroken, "two results are set aside at once");
+        if (pending_.carried()) throw Error(kBroken, "a result that added itself cannot be set aside");
+        held_ = pending_;
+        held_mark_ = parts_mark_;
+        parts_mark_ = (size_t)-1;
+        pending_ = Pending();
+        break;
       case kOpAttention:
         attention(op);
         break;
@@ -228,6 +236,7 @@ class Run {
         sample();
         break;
       case kOpAdd:
+        add_held();
         if (pending_.any() && pending_.scale != 1.f)
           ok(me_residual_add_scaled(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, pending_.scale, t_, h_,
                                     dtype_, stream_));
@@ -248,11 +257,22 @@ class Run {
   }
 
   // x += pending; out = rmsnorm(x) * w, as a kernel of its own.
+  // A result that was set aside, where the kernel at hand takes one delta only: into the stream by a kernel of its own.
+  void add_held() {
+    if (!held_.any()) return;
+    ok(me_residual_add_scaled(x_, held_.delta, held_.parts, held_.num_parts, held_.stride, held_.scale, t_, h_, dtype_, stream_));
+    held_ = Pending();
+  }
+
   void add_norm(const float* w, float eps, void* out, int groups = 1) {
-    if (groups > 1 || pending_.scale != 1.f)  // a norm in groups, or a block that multiplies what its parts give
-      ok(me_add_group_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, pending_.scale, w, out,
-                              nullptr, t_, h_, groups, eps, 1, dtype_, stream_));
-    else
+    if (held_.any() && held_.scale != pending_.scale && pending_.any()) add_held();
+    if (groups > 1 || pending_.scale != 1.f || held_.any()) {  // a norm in groups, a block that multiplies what its parts give,
+                                                              // or two parts' results at once
+      const float scale = pending_.any() ? pending_.scale : held_.scale;
+      ok(me_add_group_rmsnorm2(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, held_.delta, held_.parts,
+                               held_.num_parts, held_.stride, scale, w, out, nullptr, t_, h_, groups, eps, 1, dtype_, stream_));
+      held_ = Pending();
+    } else
       ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, w, out, nullptr, t_, h_, eps, 1,
                         dtype_, stream_));
     pending_ = Pending();
@@ -260,6 +280,12 @@ class Run {
   }
 
   void release_parts() {
+    if (held_.any()) return;  // (what was set aside lies below the pending result's memory: both go together)
+    if (held_mark_ != (size_t)-1 && !pending_.parts && !pending_.ss) {
+      arena_.used = released_to_ = std::min(held_mark_, parts_mark_);
+      held_mark_ = parts_mark_ = (size_t)-1;
+      return;
+    }
     if (parts_mark_ != (size_t)-1 && !pending_.parts && !pending_.ss) {
       arena_.used = released_to_ = parts_mark_;
       parts_mark_ = (size_t)-1;
@@ -287,7 +313,7 @@ class Run {
       release_parts();
       return;
     }
-    if (groups_of(op.i[3]) > 1 || pending_.scale != 1.f) {  // no product of this folder carries such a norm as its prologue
+    if (groups_of(op.i[3]) > 1 || pending_.scale != 1.f || held_.any()) {  // no product of this folder carries such a norm as its prologue
       add_norm(w_norm, op.f[0], normed_, groups_of(op.i[3]));
       product(normed_, op.p[1], rows_of_w, k, gated, dtype_, bufs_[op.out]);
       return;
@@ -371,7 +397,7 @@ class Run {
       pending_.stride = (long long)t_ * n;
       return;
     }
-    if (scale == 1.f && next_ && next_->kind == kOpNormLinear && next_->i[1] == h_ && groups_of(next_->i[3]) == 1 &&
+    if (scale == 1.f && !held_.any() && next_ && next_->kind == kOpNormLinear && next_->i[1] == h_ && groups_of(next_->i[3]) == 1 &&
         choose_carried_norm(dtype_, t_, n, k, (int)next_->i[0], (int)next_->i[2], compute_units(), true)) {
       // x += product in the product's epilogue, which also starts the norm behind it (choice.cpp)
       const int blocks = me_gemm_bf16_stream_carry_blocks(t_, n, k, compute_units());
@@ -385,7 +411,7 @@ class Run {
     }
     const ProductChoice c = choose_product(dtype_, kRoleDeltaInto, t_, n, k, 0, dtype_, compute_units(), true);
     if (c.adds_into) {  // x += product, in the library's epilogue: nothing stays pending
-      if (scale == 1.f && library_adds(x, op.p[1], x_, t_, n, k, stream_)) {
+      if (scale == 1.f && library_adds(x, op.p[1], x_, t_, n, k, stream_)) {  // (a result set aside waits for the next add as before)
         pending_ = Pending();
         return;
       }
@@ -568,15 +594,18 @@ class Run {
     const int rows = s_.lay.rows;
     result_.rows = rows;
     if (rows == 0) {
-      pending_ = Pending();
+      pending_ = held_ = Pending();
       return;
     }
     void* picked = arena_.take((size_t)rows * h_ * elem_);
-    if (groups_of(op.i[0]) > 1 || pending_.scale != 1.f)
-      ok(me_add_group_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, pending_.scale,
-                              (const float*)op.p[0], picked, idx(s_.lay.want_rows), rows, h_, groups_of(op.i[0]), op.f[0], 0, dtype_,
-                              stream_));
-    else
+    if (held_.any() && held_.scale != pending_.scale && pending_.any()) add_held();
+    if (groups_of(op.i[0]) > 1 || pending_.scale != 1.f || held_.any()) {
+      const float scale = pending_.any() ? pending_.scale : held_.scale;
+      ok(me_add_group_rmsnorm2(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, held_.delta, held_.parts,
+                               held_.num_parts, held_.stride, scale, (const float*)op.p[0], picked, idx(s_.lay.want_rows), rows, h_,
+                               groups_of(op.i[0]), op.f[0], 0, dtype_, stream_));
+      held_ = Pending();
+    } else
       ok(me_add_rmsnorm(x_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, (const float*)op.p[0], picked,
                         idx(s_.lay.want_rows), rows, h_, op.f[0], 0, dtype_, stream_));
     pending_ = Pending();
@@ -636,7 +665,8 @@ class Run {
   float *x_, *spare_;
   void* normed_;
   std::vector<void*> bufs_;
-  Pending pending_;
+  Pending pending_, held_;  // held_: a result set aside (kOpHold) until the add that takes it together with pending_
+  size_t held_mark_ = (size_t)-1;
   struct AttnParts {  // what a decode attention left for the output projection behind it
     float *o = nullptr, *ml = nullptr;
     int splits = 0, nh = 0, d = 0, value = -1;

@@ -48,6 +48,8 @@ enum OpKind {
                       // i0 heads, i1 d, i2 dv, i3 rotary size, i4 pairing, i5 activation of q, k, v, i6 kind of the output norm,
                       // i7 activation of the gate, i8 positions the table covers; f0 scale on k, f1 eps
                       // -> out [tokens, heads * dv]
+  kOpHold = 13,       // the pending delta is set aside until the next add: a second part that reads the same normed input
+                      // follows, and the add takes both results at once (with the same multiplier)
 };
 
 constexpr int kOpInts = 16, kOpFloats = 4;

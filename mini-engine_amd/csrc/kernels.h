@@ -38,6 +38,10 @@ int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const float* k_w, c
 int me_add_group_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, float delta_scale,
                          const float* w, void* h, const int* rows, int num_rows, int dim, int groups, float eps, int write_x,
                          int dtype, hipStream_t stream);
+int me_add_group_rmsnorm2(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, const void* delta2,
+                          const float* parts2, int num_parts2, long long part_stride2, float delta_scale, const float* w, void* h,
+                          const int* rows, int num_rows, int dim, int groups, float eps, int write_x, int dtype,
+                          hipStream_t stream);
 int me_residual_add_scaled(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, float scale,
                            int num_rows, int dim, int dtype, hipStream_t stream);
 int me_decay_state_padded_dim(int d);

@@ -28,7 +28,7 @@ from ..ops.library import lib
 _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 _declared = False
 
-EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS, DECAY_STATE = range(13)
+EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS, DECAY_STATE, HOLD = range(14)
 OP_INTS, OP_FLOATS = 16, 4  # csrc/host/program.h: kOpInts, kOpFloats
 _RAISES = {1: ValueError, 2: RuntimeError, 3: AssertionError}
 
@@ -150,6 +150,7 @@ class StepProgram:
         self._value_kinds: list[tuple[int, int]] = []
         self._scopes: list[list[int]] = []
         self._pending_value: int | None = None
+        self._held_value: int | None = None  # the value of a delta that was set aside (hold)
         self.num_ops = 0
         self.delta_scale = 1.0  # what the block being written multiplies its parts' results by (set by the block)
         self.draws = False
@@ -190,16 +191,17 @@ class StepProgram:
             yield
         finally:
             for v in self._scopes.pop():
-                if v != self._pending_value:
+                if v != self._pending_value and v != self._held_value:
                     self._give_back(v)
 
     def _give_back(self, v: int) -> None:
         self._free[self._value_kinds[v]].append(v)
 
     def pending_consumed(self) -> None:
-        v, self._pending_value = self._pending_value, None
-        if v is not None and not any(v in s for s in self._scopes):
-            self._give_back(v)
+        for v in (self._pending_value, self._held_value):
+            if v is not None and not any(v in s for s in self._scopes):
+                self._give_back(v)
+        self._pending_value = self._held_value = None
 
     # -------------------------------------------------------------- operations
     def op(self, kind: int, in_: int = -1, out: int = -1, ptrs=(), ints=(), floats=()) -> None:
@@ -331,6 +333,12 @@ class StepProgram:
         """The pending delta into the residual stream, as a kernel of its own (before a norm that is not RMS-shaped)."""
         self.op(ADD)
         self.pending_consumed()
+
+    def hold(self) -> None:
+        """The pending delta is set aside: another part that reads the same normed input follows, and the next add (of
+        the next norm, of the head, or a kernel of its own) takes both results at once."""
+        self.op(HOLD)
+        self._held_value, self._pending_value = self._pending_value, None
 
     def call(self, fn, in_: int = -1, out_cols: int | None = None, out_elem: int | None = None) -> int:
         """A part with code of its own: when a step reaches this place, ``fn(frame)`` is called with a

@@ -65,8 +65,8 @@ class PreNormBlock:
 
 class ParallelBlock:
     """One norm; the mixer and the feed-forward both read its output; their sum, times the spec's ``residual_scale``,
-    is added to the stream. The mixer's result is added by a kernel of its own (the feed-forward does not wait for it:
-    it reads the normed activations); the feed-forward's stays pending for the next norm, like a pre-norm block's."""
+    is added to the stream. The mixer's result is set aside while the feed-forward runs (it reads the normed
+    activations, not the stream); the next norm adds both results, scaled, while it norms."""
 
     def __init__(self, spec, dtype: torch.dtype, device: torch.device):
         self.spec, self.dtype = spec, dtype
@@ -108,7 +108,7 @@ class ParallelBlock:
                     if out is not None:
                         program.delta(out)
                     if at + 1 < len(parts):
-                        program.add()  # the last part's result waits for the next norm instead
+                        program.hold()  # set aside: the next norm's kernel adds it together with the last part's result
             finally:
                 program.delta_scale = before
 
