@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256) void decay_state_chunk_starts_kernel(float* __
 // 1: all heads' outputs together over sqrt(mean^2 + eps), times w [heads * dv]. Then times act(gate), where the gate
 // is the last heads * dv columns of the projections.
 template <typename T>
-__global__ __launch_bounds__(256) void decay_state_finish_kernel(const float* __restrict__ o32, const T* __restrict__ proj,
+__global__ __launch_bounds__(1024) void decay_state_finish_kernel(const float* __restrict__ o32, const T* __restrict__ proj,
                                                                   int proj_cols, int gate_at, const float* __restrict__ w,
                                                                   T* __restrict__ out, int heads, int dv, int norm_kind,
                                                                   int gate_act, float eps) {
@@ -287,12 +287,18 @@ __global__ __launch_bounds__(256) void decay_state_finish_kernel(const float* __
       ss = wave_sum(ss);
       if (lane == 0) inv[h] = rsqrtf(ss / (float)dv + eps);
     }
-  } else {  // a wave adds up the whole row: the order follows from its length alone
-    if (wave == 0) {
-      float ss = 0.f;
-      for (int i = lane; i < n; i += ME_WAVE) ss = fmaf(orow[i], orow[i], ss);
-      ss = wave_sum(ss);
-      if (lane == 0) inv[0] = rsqrtf(ss / (float)n + eps);
+  } else {  // every wave adds up a stretch of the row, the stretches' sums are added in their order: the order of the
+            // whole sum follows from the row's length and the block's size, which follows from the sizes too
+    const int stretch = (n + waves - 1) / waves;
+    float ss = 0.f;
+    for (int i = wave * stretch + lane; i < min((wave + 1) * stretch, n); i += ME_WAVE) ss = fmaf(orow[i], orow[i], ss);
+    ss = wave_sum(ss);
+    if (lane == 0) inv[1 + wave] = ss;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float total = 0.f;
+      for (int w = 0; w < waves; ++w) total += inv[1 + w];
+      inv[0] = rsqrtf(total / (float)n + eps);
     }
   }
   __syncthreads();
@@ -372,6 +378,7 @@ extern "C" int me_decay_state(const void* proj, const float* rope_table, int rd,
   const dim3 scan_grid2(scan_grid.x, heads, (dv + 127) / 128);  // two columns a lane
   if (scan_grid.z > 65535 || (long long)d * dv > (1ll << 24)) return me_fail("me_decay_state: value heads of %d elements", dv);
   const dim3 starts_grid((d * dv + 255) / 256, heads, items);
+  const int finish_threads = heads * dv >= 1024 * 2 && heads >= 16 ? 1024 : heads * dv >= 512 * 2 && heads >= 8 ? 512 : 256;
 #define DS_SCAN_MODE(RPL, MODE)                                                                                              \
   do {                                                                                                                       \
     int failed;                                                                                                              \
@@ -407,7 +414,8 @@ extern "C" int me_decay_state(const void* proj, const float* rope_table, int rd,
       DS_SCAN(32);                                                                                                          \
     else                                                                                                                    \
       DS_SCAN(64);                                                                                                          \
-    decay_state_finish_kernel<T><<<num_tokens, 256, 0, stream>>>(o32, (const T*)proj, proj_cols, 2 * heads * d + heads * dv, \
+    /* a wave a head where a block can have that many: a head's sum is one trip to memory, not one per round of the waves */ \
+    decay_state_finish_kernel<T><<<num_tokens, finish_threads, 0, stream>>>(o32, (const T*)proj, proj_cols, 2 * heads * d + heads * dv, \
                                                                  norm_w, (T*)out, heads, dv, norm_kind, gate_act, eps);      \
   } while (0)
   if (dtype == ME_F32)
