@@ -746,7 +746,7 @@ extern "C" int me_qk_norm_rope_scatter(const void* qkv, const float* q_w, const 
 // One block per row, a wave per group at a time: a group's sum of squares is added up in an order that its length
 // alone fixes. groups == 1 and delta_scale == 1 is the norm of the kernels above. A second delta (`delta2` or `parts2`,
 // the result of a part that ran beside the first on the same normed input) is added with the same scale.
-#define ME_MAX_NORM_GROUPS 64
+#define ME_MAX_NORM_GROUPS 1024
 
 template <typename T>
 __global__ void add_group_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ parts,

@@ -35,7 +35,8 @@ class Attention(Mixer):
         super().__init__(spec, dtype, device)
         s = spec
         if not (float(s.scale) > 0.0 and float(s.scale) < float("inf")):
-            raise ValueError(f"the score scale must be positive and finite, got {s.scale}: the kernels scale before they mask")
+            raise ValueError(f"the score scale must be positive and finite, got {s.scale}: the matrix-core kernels take a "
+                             f"tile's maximum before they scale")
         if s.num_heads % s.num_kv_heads:
             raise ValueError(f"{s.num_heads} query heads are not a multiple of {s.num_kv_heads} key/value heads")
         if s.window < 0:

@@ -55,10 +55,16 @@ def configs() -> dict[str, dict]:
             attention(4, 2, 64, 64, 50, 6, 32, 1e4, 0.125, ff=128),
             lightning(2, 32, 32, (0.9, 0.99)),
             attention(8, 8, 32, 32, 100, 70, 32, 1e5, 0.2, ff=128)]),
+        # sizes that are no multiple of 8 (products of this folder's kernels that take any size), five norm groups,
+        # layers without a feed-forward
+        "T": model(211, 100, 5, 0.9, 1e-4, [
+            lightning(3, 12, 20, (0.9, 0.5, 0.99)),
+            attention(5, 1, 20, 28, 9, 2, 10, 77.0, 0.4),
+            retention(2, 36, 10, (0.95, 0.999), 36, 1e4, ff=52)]),
     }
 
 
-BLOCK_SIZES = {"P": 16, "Q": 32, "R": 8, "S": 16}
+BLOCK_SIZES = {"P": 16, "Q": 32, "R": 8, "S": 16, "T": 16}
 
 
 def write_folder(folder: str, cfg: dict, seed: int = 0, std: float = 0.08) -> str:
