@@ -811,8 +811,8 @@ static inline int gs_of(int dim, int groups) { return dim / groups; }
 // the row, 64 threads apart, so every load of a row (the stream, both deltas, all partial sums, the weight) is asked for at
 // once; a wave's 64 consecutive elements lie in one group and give one partial sum of squares, and a group's sum is its
 // runs' sums added in the order of the runs (a function of the row's length and the groups alone, whatever the block's
-// size). One item's row of 1,024 behind ten partial sums: 12 us with a wave a group and eight elements a lane in turn,
-// 4 us this way.
+// size). One item's row of 1,024 behind ten partial sums: 12.3 us with a wave a group and eight elements a lane in turn,
+// 6.0 us this way.
 template <typename T>
 __global__ __launch_bounds__(1024) void add_group_rmsnorm_wide_kernel(
     float* __restrict__ x, const T* __restrict__ delta, const float* __restrict__ parts, int num_parts, size_t part_stride,
@@ -886,7 +886,9 @@ extern "C" int me_add_group_rmsnorm2(void* x, const void* delta, const float* pa
   if (parts && (num_parts < 1 || part_stride < (long long)dim)) return me_fail("me_add_group_rmsnorm: %d partial sums", num_parts);
   if (parts2 && (num_parts2 < 1 || part_stride2 < (long long)dim)) return me_fail("me_add_group_rmsnorm: %d partial sums", num_parts2);
   if (gs_of(dim, groups) % ME_WAVE == 0 && dim <= 4096) {  // whole runs of 64 elements: a thread an element (up to four)
-    const int wide = dim <= 1024 ? dim : 1024;  // (a multiple of 64)
+    // (a multiple of 64) few rows: a thread an element, a row's loads all at once; many rows: four elements a thread (the
+    // 2,048 rows of a prompt, width 1,024, two partial sums: 29.5 us in blocks of 1,024 threads, 17.2 in blocks of 256)
+    const int wide = num_rows >= 128 && dim >= 256 ? ((dim / 4 + 63) / 64) * 64 : (dim <= 1024 ? dim : 1024);
     if (dtype == ME_F32)
       add_group_rmsnorm_wide_kernel<float><<<num_rows, wide, 0, stream>>>(
           (float*)x, (const float*)delta, parts, num_parts, (size_t)part_stride, (const float*)delta2, parts2, num_parts2,
