@@ -482,7 +482,8 @@ template <typename T>
 __device__ __forceinline__ void v_scatter_segment(VScatterLds<T>& lds, int segment, int kvh, const T* __restrict__ qkv,
                                                   const int* __restrict__ positions, const int* __restrict__ item_start,
                                                   int num_items, const int* __restrict__ block_table, int table_width,
-                                                  T* __restrict__ v_cache, int nh, int nkv, int d, int bs) {
+                                                  T* __restrict__ v_cache, int nh, int nkv, int d, int bs,
+                                                  const float* __restrict__ turn_table = nullptr, int turn_pairing = 0) {
   T(&tile)[16][ME_MAX_HEAD_DIM + 2] = lds.tile;
   int& s_item = lds.item;
   int& s_seg = lds.seg;
@@ -520,6 +521,20 @@ __device__ __forceinline__ void v_scatter_segment(VScatterLds<T>& lds, int segme
       tile[first - seg_pos + row][col] = src[(size_t)(t0 + first - p0 + row) * width + col];
     }
   }
+  if (turn_table) {  // values that are cached turned by their own position: pair j of a row by the angles of its position
+    __syncthreads();
+    const int half = d / 2;
+    for (int idx = threadIdx.x; idx < (last - first + 1) * half; idx += blockDim.x) {
+      const int row = idx / half, j = idx % half;
+      const float* cs = turn_table + (size_t)(first + row) * d;  // [2, d / 2] of the row's position
+      const float c = cs[j], sn = cs[half + j];
+      const int a = turn_pairing == 0 ? j : 2 * j, b = turn_pairing == 0 ? j + half : 2 * j + 1;
+      T(&trow)[ME_MAX_HEAD_DIM + 2] = tile[first - seg_pos + row];
+      const float u = to_float(trow[a]), v = to_float(trow[b]);
+      trow[a] = from_float<T>(u * c - v * sn);
+      trow[b] = from_float<T>(v * c + u * sn);
+    }
+  }
   __syncthreads();
   const int page = block_table[(size_t)item * table_width + seg_pos / bs];
   if (page < 0) return;
@@ -545,10 +560,12 @@ template <typename T>
 __global__ __launch_bounds__(256) void v_scatter_tiles_kernel(const T* __restrict__ qkv, const int* __restrict__ positions,
                                                               const int* __restrict__ item_start, int num_items,
                                                               const int* __restrict__ block_table, int table_width,
-                                                              T* __restrict__ v_cache, int nh, int nkv, int d, int bs) {
+                                                              T* __restrict__ v_cache, int nh, int nkv, int d, int bs,
+                                                              const float* __restrict__ turn_table = nullptr,
+                                                              int turn_pairing = 0) {
   __shared__ VScatterLds<T> lds;
   v_scatter_segment<T>(lds, blockIdx.x, blockIdx.y, qkv, positions, item_start, num_items, block_table, table_width,
-                       v_cache, nh, nkv, d, bs);
+                       v_cache, nh, nkv, d, bs, turn_table, turn_pairing);
 }
 
 // The same work for the common geometry (head size a power of two from 16 to 256, rotary over the
@@ -979,11 +996,11 @@ __global__ __launch_bounds__(256) void qkv_rotate_scatter_kernel(
     const float* __restrict__ rope_table, int rd, int pairing, const float* __restrict__ v_table, int v_pairing,
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
     int table_width, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int nkv, int d, int dv,
-    int bs, float eps, int heads_per_block) {
+    int bs, float eps, int heads_per_block, int skip_v) {
   __shared__ float stage[4][ME_MAX_HEAD_DIM];
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int t = blockIdx.x;
-  const int heads_total = nh + 2 * nkv;
+  const int heads_total = skip_v ? nh + nkv : nh + 2 * nkv;  // (value heads may be written by the page-tile kernel)
   const size_t width = (size_t)(nh + nkv) * d + (size_t)nkv * dv;
   const int pos = positions[t];
   const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
@@ -1061,11 +1078,14 @@ __global__ __launch_bounds__(256) void qkv_rotate_scatter_kernel(
   }
 }
 
-extern "C" int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd,
-                                     int pairing, const float* v_table, int v_pairing, const int* positions,
-                                     const int* token_item, const int* block_table, int table_width, void* q_out,
-                                     void* k_cache, void* v_cache, int num_tokens, int nh, int nkv, int d, int dv, int bs,
-                                     float eps, int dtype, hipStream_t stream) {
+// item_start / num_items / num_segments: when given (num_segments > 0: the sum over items of (pos0 + qlen - 1)/16 - pos0/16
+// + 1) and the values have the keys' size, the values are turned and written a page segment of 16 slots at a time.
+extern "C" int me_qkv_rotate_scatter_tiles(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd,
+                                           int pairing, const float* v_table, int v_pairing, const int* positions,
+                                           const int* token_item, const int* block_table, int table_width, void* q_out,
+                                           void* k_cache, void* v_cache, int num_tokens, int nh, int nkv, int d, int dv, int bs,
+                                           float eps, int dtype, const int* item_start, int num_items, int num_segments,
+                                           hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (d <= 0 || d > ME_MAX_HEAD_DIM || dv <= 0 || dv > ME_MAX_HEAD_DIM)
     return me_fail("me_qkv_rotate_scatter: head sizes %d and %d must be in 1..%d", d, dv, ME_MAX_HEAD_DIM);
@@ -1074,19 +1094,39 @@ extern "C" int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const fl
   if ((pairing | v_pairing) & ~1) return me_fail("me_qkv_rotate_scatter: pairing is 0 (halves) or 1 (neighbours)");
   if (nh <= 0 || nkv <= 0 || bs <= 0 || table_width <= 0)
     return me_fail("me_qkv_rotate_scatter: nh=%d nkv=%d block_size=%d table_width=%d", nh, nkv, bs, table_width);
-  const int heads_total = nh + 2 * nkv;
+  const bool tiles = num_segments > 0 && item_start != nullptr && num_items > 0 && dv == d && bs % 16 == 0 && nkv <= 65535;
+  const int heads_total = tiles ? nh + nkv : nh + 2 * nkv;
   const int hpb = num_tokens >= 512 ? 8 : 4;  // heads a block of four waves takes, a wave a head at a time
   dim3 grid(num_tokens, (heads_total + hpb - 1) / hpb);
   if (grid.y > 65535) return me_fail("me_qkv_rotate_scatter: too many heads");
-  if (dtype == ME_F32)
+  if (dtype == ME_F32) {
     qkv_rotate_scatter_kernel<float><<<grid, 256, 0, stream>>>(
         (const float*)qkv, q_w, k_w, rope_table, rd, pairing, v_table, v_pairing, positions, token_item, block_table, table_width,
-        (float*)q_out, (float*)k_cache, (float*)v_cache, nh, nkv, d, dv, bs, eps, hpb);
-  else
+        (float*)q_out, (float*)k_cache, (float*)v_cache, nh, nkv, d, dv, bs, eps, hpb, tiles ? 1 : 0);
+    if (tiles)
+      v_scatter_tiles_kernel<float><<<dim3(num_segments, nkv), 256, 0, stream>>>(
+          (const float*)qkv, positions, item_start, num_items, block_table, table_width, (float*)v_cache, nh, nkv, d, bs, v_table,
+          v_pairing);
+  } else {
     qkv_rotate_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(
         (const bf16_t*)qkv, q_w, k_w, rope_table, rd, pairing, v_table, v_pairing, positions, token_item, block_table, table_width,
-        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, dv, bs, eps, hpb);
+        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, dv, bs, eps, hpb, tiles ? 1 : 0);
+    if (tiles)
+      v_scatter_tiles_kernel<bf16_t><<<dim3(num_segments, nkv), 256, 0, stream>>>(
+          (const bf16_t*)qkv, positions, item_start, num_items, block_table, table_width, (bf16_t*)v_cache, nh, nkv, d, bs, v_table,
+          v_pairing);
+  }
   return me_check_launch("me_qkv_rotate_scatter");
+}
+
+extern "C" int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd,
+                                     int pairing, const float* v_table, int v_pairing, const int* positions,
+                                     const int* token_item, const int* block_table, int table_width, void* q_out,
+                                     void* k_cache, void* v_cache, int num_tokens, int nh, int nkv, int d, int dv, int bs,
+                                     float eps, int dtype, hipStream_t stream) {
+  return me_qkv_rotate_scatter_tiles(qkv, q_w, k_w, rope_table, rd, pairing, v_table, v_pairing, positions, token_item, block_table,
+                                     table_width, q_out, k_cache, v_cache, num_tokens, nh, nkv, d, dv, bs, eps, dtype, nullptr, 0, 0,
+                                     stream);
 }
 
 // ---------------------------------------------------------------- rows turned back by their positions' angles

@@ -462,8 +462,12 @@ class Run {
       const int v_pairing = op.i[12] ? (int)op.i[12] - 1 : 0;
       if (!owns) throw Error(kBadValue, "an attention layer of this form writes its own pages");
       void* q = arena_.take((size_t)t_ * nh * d * elem_);
-      ok(me_qkv_rotate_scatter(qkv, q_w, k_w, rope, rd, pairing, v_table, v_pairing, idx(s_.lay.positions), idx(s_.lay.token_item),
-                               table, width, q, kc, vc, t_, nh, nkv, d, dv, bs, eps, dtype_, stream_));
+      int segments = 0;
+      if (t_ >= 64 && dv == d)  // many tokens: the values are turned and written a page segment (a transposed tile) at a time
+        for (int i = 0; i < items; ++i) segments += (s_.starts[i] + s_.qlens[i] - 1) / 16 - s_.starts[i] / 16 + 1;
+      ok(me_qkv_rotate_scatter_tiles(qkv, q_w, k_w, rope, rd, pairing, v_table, v_pairing, idx(s_.lay.positions),
+                                     idx(s_.lay.token_item), table, width, q, kc, vc, t_, nh, nkv, d, dv, bs, eps, dtype_,
+                                     segments ? idx(s_.lay.item_start) : nullptr, items, segments, stream_));
       if (s_.decode_only && attention_takes_tiled_prefill(op, dtype_)) {
         // one new token per item: the split-context kernel, which deals the kept first keys' tiles to its splits before
         // the window's; a second kernel (or the blocks themselves) adds up the splits

@@ -35,6 +35,11 @@ int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const float* k_w, c
                           const float* v_table, int v_pairing, const int* positions, const int* token_item,
                           const int* block_table, int table_width, void* q_out, void* k_cache, void* v_cache, int num_tokens,
                           int nh, int nkv, int d, int dv, int bs, float eps, int dtype, hipStream_t stream);
+int me_qkv_rotate_scatter_tiles(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd, int pairing,
+                                const float* v_table, int v_pairing, const int* positions, const int* token_item,
+                                const int* block_table, int table_width, void* q_out, void* k_cache, void* v_cache,
+                                int num_tokens, int nh, int nkv, int d, int dv, int bs, float eps, int dtype,
+                                const int* item_start, int num_items, int num_segments, hipStream_t stream);
 int me_add_group_rmsnorm(void* x, const void* delta, const float* parts, int num_parts, long long part_stride, float delta_scale,
                          const float* w, void* h, const int* rows, int num_rows, int dim, int groups, float eps, int write_x,
                          int dtype, hipStream_t stream);

@@ -280,11 +280,15 @@ def _check_cache(k_cache, v_cache, dtype, nkv, d, bs, dv=None):
 
 
 def qkv_rotate_scatter(qkv, q_w, k_w, rope, pairing, v_table, v_pairing, positions, token_item, block_table, k_cache, v_cache,
-                       nh: int, nkv: int, d: int, dv: int, eps: float, q_out: torch.Tensor | None = None) -> torch.Tensor:
+                       nh: int, nkv: int, d: int, dv: int, eps: float, q_out: torch.Tensor | None = None,
+                       item_start: torch.Tensor | None = None, starts: list[int] | None = None,
+                       qlens: list[int] | None = None) -> torch.Tensor:
     """Per-head q/k norm (``q_w`` / ``k_w`` float32 [d] or None), rotation of the first elements of q and k by the angles
     of ``rope`` [P, 2, r/2] (``pairing`` 0: j with j + r/2; 1: 2j with 2j + 1), values turned over all ``dv`` elements by
     ``v_table`` [P, 2, dv/2] (or copied), keys and values written to their pages. ``qkv`` is ``[T, nh d + nkv d + nkv dv]``;
-    returns q ``[T, nh, d]``. Every position must lie inside the tables and in a page of the token's table row."""
+    returns q ``[T, nh, d]``. Every position must lie inside the tables and in a page of the token's table row. With
+    ``item_start`` (int32 [items + 1]) and the items' first positions and lengths on the host, values of the keys' size
+    are turned and written a page segment of 16 slots at a time."""
     _want(qkv, "qkv", None, (None, nh * d + nkv * (d + dv)))
     t = qkv.shape[0]
     bs = k_cache.shape[2]
@@ -302,10 +306,16 @@ def qkv_rotate_scatter(qkv, q_w, k_w, rope, pairing, v_table, v_pairing, positio
     if q_out is None:
         q_out = torch.empty((t, nh, d), dtype=qkv.dtype, device=qkv.device)
     _want(q_out, "q_out", qkv.dtype, (t, nh, d))
-    check(lib().me_qkv_rotate_scatter(_p(qkv), _p(q_w), _p(k_w), _p(rope), _i(rd), _i(pairing), _p(v_table), _i(v_pairing),
-                                      _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]), _p(q_out),
-                                      _p(k_cache), _p(v_cache), _i(t), _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _f(eps),
-                                      _i(_code(qkv.dtype)), _stream()))
+    segments = items = 0
+    if item_start is not None and starts is not None and qlens is not None and dv == d:
+        items = len(qlens)
+        _want(item_start, "item_start", torch.int32, (items + 1,))
+        segments = sum((s + n - 1) // 16 - s // 16 + 1 for s, n in zip(starts, qlens))
+    check(lib().me_qkv_rotate_scatter_tiles(_p(qkv), _p(q_w), _p(k_w), _p(rope), _i(rd), _i(pairing), _p(v_table), _i(v_pairing),
+                                            _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]), _p(q_out),
+                                            _p(k_cache), _p(v_cache), _i(t), _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _f(eps),
+                                            _i(_code(qkv.dtype)), _p(item_start if segments else None), _i(items), _i(segments),
+                                            _stream()))
     return q_out
 
 

@@ -183,7 +183,9 @@ def test_tiled_prompt_attention_sees_the_kept_first_keys(nh, nkv, d, rd, pairing
         item = torch.cat([torch.full((n,), i) for i, n in enumerate(qlens)]).to(torch.int32).cuda()
         item_start = torch.tensor([0, qlens[0], sum(qlens)], dtype=torch.int32).cuda()
         rows = torch.cat([seqs[i][lo:hi] for i, (lo, hi) in enumerate(cuts)]).cuda().contiguous()
-        q = K.qkv_rotate_scatter(rows, None, None, rope, code, vt, code, pos, item, table, k_cache, v_cache, nh, nkv, d, d, eps)
+        # (the values go to their pages a segment of 16 slots at a time)
+        q = K.qkv_rotate_scatter(rows, None, None, rope, code, vt, code, pos, item, table, k_cache, v_cache, nh, nkv, d, d, eps,
+                                 item_start=item_start, starts=starts, qlens=qlens)
         out = K.attention_prefill_bf16(q, k_cache, v_cache, pos, item_start, qlens, table, scale, size, starts=starts,
                                        keep_first=keep)
         K.unturn_rows(out, vt, code, pos, nh)
