@@ -26,6 +26,7 @@ class NormSpec:
     eps: float
     kind: str = "rmsnorm"
     groups: int = 1
+    weight_offset: float = 0.0  # the stored weight lies this far below the one that multiplies (1.0: weights stored around zero)
 
 
 @dataclass(frozen=True)
@@ -42,6 +43,27 @@ class RotarySpec:
     kind: str = "rotary"
     pairing: str = "halves"
     angles: str = "float32"
+
+
+@dataclass(frozen=True)
+class YarnRotarySpec:
+    """Rotary encoding over pairs of halves whose slow frequencies are stretched for contexts beyond the ``original`` one.
+
+    With ``f_j = theta ** (-2j / rotary_dim)`` and ``dim(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta)`` (the
+    pair that makes ``t`` turns over the original context), ``lo = max(floor(dim(fast)), 0)``, ``hi = min(ceil(dim(slow)),
+    rotary_dim - 1)``, ``ramp_j = clamp((j - lo) / max(hi - lo, 0.001), 0, 1)``: pair j turns at
+    ``f_j / factor * ramp_j + f_j * (1 - ramp_j)``, and cosines and sines are multiplied by ``0.1 * ln(factor) + 1``. The
+    table is worked out in double precision and rounded once.
+    """
+
+    rotary_dim: int
+    theta: float
+    factor: float
+    original: float
+    fast: float
+    slow: float
+    kind: str = "yarn_rotary"
+    pairing: str = "halves"
 
 
 @dataclass(frozen=True)
@@ -74,6 +96,12 @@ class AttentionSpec:
     keep_first: int = 0
     value_position: Any | None = None
     names: tuple[tuple[str, str], ...] = ()
+    # q and k are divided by their root mean square per head without a weight (with ``qk_norm_eps``)
+    qk_norm_weight: bool = True
+    # (coef, every) or None: the query at position p is multiplied by 1 + coef * ln(floor((p + 1) / every) + 1)
+    query_temperature: tuple[float, int] | None = None
+    # a projection to one number per head (role ``g`` of ``names``) whose sigmoid multiplies the head's output
+    output_gate: bool = False
 
     @property
     def v_dim(self) -> int:
@@ -83,6 +111,39 @@ class AttentionSpec:
     def kv_elements_per_token(self) -> int:
         """Key and value elements one token occupies in this layer's own pages (none when it reads another's)."""
         return 0 if self.cache_from is not None else self.num_kv_heads * (self.head_dim + self.v_dim)
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Causal attention whose keys and values are linear maps of one latent per token.
+
+    A token's projection gives ``latent_rank`` elements, RMS-normed with a weight: the latent c; and ``rotary_dim`` more, turned
+    by the position: a key part that all heads share. Head h has the key ``[W_uk_h c | shared part]`` and the value
+    ``W_uv_h c``; its query has ``head_dim`` elements that meet the first part and ``rotary_dim`` turned ones that meet the
+    second. Only the latent and the shared part are cached. ``sink``: a learned logit per head that counts once in the
+    softmax's denominator and has no value. ``output_gate`` as in :class:`AttentionSpec`. ``names`` maps the roles ``q dkv
+    dkv_norm uk uv sink g o`` to the checkpoint's suffixes.
+    """
+
+    hidden_size: int
+    num_heads: int
+    head_dim: int
+    rotary_dim: int
+    value_dim: int
+    latent_rank: int
+    scale: float
+    norm_eps: float
+    position: Any
+    sink: bool = False
+    output_gate: bool = False
+    names: tuple[tuple[str, str], ...] = ()
+    kind: str = "latent_attention"
+
+    @property
+    def kv_elements_per_token(self) -> int:
+        """Elements one token occupies in this layer's pages: the key ``[c | shared part]`` and its value rows, the latent
+        once more."""
+        return 2 * self.latent_rank + self.rotary_dim
 
 
 @dataclass(frozen=True)
@@ -129,12 +190,39 @@ class GatedMlpSpec:
 
 
 @dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """A feed-forward of ``num_experts`` gated feed-forwards of ``intermediate_size`` each, of which a token uses the ``top_k``
+    with the largest router logits (float32), weighted by the softmax over those logits alone. Tensors: ``<prefix>.<router>``
+    ``[experts, hidden]`` and ``<prefix>.<expert><e>.<gate|up|down>``; ``names`` maps the roles ``router expert gate up down``."""
+
+    hidden_size: int
+    intermediate_size: int
+    num_experts: int
+    top_k: int
+    activation: str = "silu"
+    names: tuple[tuple[str, str], ...] = ()
+    kind: str = "routed_experts"
+
+
+@dataclass(frozen=True)
+class HyperConnectionSpec:
+    """How a part of a layer is tied to ``streams`` residual streams: it reads ``sum_s in[s] x_s``, and once it has given y
+    every stream is rewritten from the old ones, ``x_t = sum_s mix[s, t] x_s + out[t] y``. ``prefix`` names the tensors
+    ``<prefix>.in [streams]``, ``<prefix>.out [streams]`` and ``<prefix>.mix [streams, streams]``."""
+
+    streams: int
+    prefix: str
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One residual block: which mixer, which feed-forward, which norms, and how they are arranged.
 
     ``arrangement == "pre_norm"``: ``x += mixer(norm1(x)); x += ffn(norm2(x))``.
     ``arrangement == "parallel"``: ``h = norm1(x); x += residual_scale * (mixer(h) + ffn(h))``: one norm (``mixer_norm``)
     that both parts read; ``ffn`` may be None (then ``ffn_norm`` and its names are not used).
+    ``arrangement == "hyper_connections"``: as ``pre_norm`` over several residual streams: each part reads and rewrites them by
+    its :class:`HyperConnectionSpec` (``mixer_streams``, ``ffn_streams``); ``ffn`` may be None.
     The ``*_prefix`` / ``*_name`` strings are the checkpoint names of this layer's tensors.
     """
 
@@ -148,6 +236,8 @@ class LayerSpec:
     ffn_norm_name: str
     arrangement: str = "pre_norm"
     residual_scale: float = 1.0
+    mixer_streams: Any | None = None
+    ffn_streams: Any | None = None
 
 
 @dataclass(frozen=True)
@@ -168,6 +258,7 @@ class ModelPlan:
     eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
     embedding_multiplier: float | None = None  # the looked-up rows are multiplied by it (None: as they are)
     logit_scale: float | None = None  # the logits are multiplied by it (None: as they are)
+    residual_streams: int = 0  # > 0: that many residual streams, all the embedding at first, summed before the final norm
 
     def __post_init__(self) -> None:
         n = len(self.layers)

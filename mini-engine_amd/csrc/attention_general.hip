@@ -45,7 +45,8 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
     int table_width, T* __restrict__ out, int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
-    const float* __restrict__ unturn, int un_pairing, float scale, int wpu) {
+    const float* __restrict__ unturn, int un_pairing, float scale, int wpu, const float* __restrict__ sink,
+    const T* __restrict__ gate, size_t gate_row) {
   constexpr int KMAX = AG_MAX_D / ME_WAVE;
   __shared__ float qs[8][AG_MAX_D];
   __shared__ float parts[8][AG_MAX_D + 2];  // with several waves per unit: a round's results (values, maximum, sum)
@@ -208,7 +209,14 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
   }
   if (w != 0) return;
   T* orow = out + ((size_t)t * nh + head) * dv;
-  const float inv = 1.f / lt;
+  if (sink) {  // one more term exp(sink) in the denominator, with no value: a chunk of its own, merged last
+    float none[KMAX];
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) none[k] = 0.f;
+    ag_merge<KMAX>(mt, lt, acct, sink[head], 1.f, none);
+  }
+  float inv = 1.f / lt;
+  if (gate) inv *= 1.f / (1.f + expf(-to_float(gate[(size_t)t * gate_row + head])));  // the head's output gate
   if (unturn) {  // the sum of turned values, turned back by this token's angles: through this wave's row of LDS
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -446,18 +454,22 @@ __global__ __launch_bounds__(1024) void attention_shared_f32_kernel(
 // dv: size of the value heads (out is [tokens, nh * dv]); keep_first: the first keys that stay visible behind the window;
 // unturn (float32 [positions, 2, dv/2] or null) and un_pairing (0: element j with j + dv/2; 1: 2j with 2j + 1): the
 // angles that every output row is turned back by. Steps with any of these go to the first kernel.
-extern "C" int me_attention_general_ext(const void* q, const void* k_cache, const void* v_cache, const int* positions,
-                                        const int* token_item, const int* block_table, int table_width, void* out,
-                                        int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
-                                        const float* unturn, int un_pairing, float scale, int dtype, int items,
-                                        hipStream_t stream) {
+//
+// sink (float32 [nh] or null): a learned logit per head that counts once in the softmax's denominator and has no value (it
+// is not multiplied by the scale). gate (or null; gate[t * gate_row + head] in the activations' type): every head's output
+// is multiplied by the sigmoid of its gate before it is rounded.
+extern "C" int me_attention_general_gated(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                                          const int* token_item, const int* block_table, int table_width, void* out,
+                                          int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
+                                          const float* unturn, int un_pairing, float scale, const float* sink, const void* gate,
+                                          long long gate_row, int dtype, int items, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
   if (d <= 0 || d > AG_MAX_D) return me_fail("me_attention_general: head_dim=%d must be in 1..%d", d, AG_MAX_D);
   if (dv <= 0 || dv > AG_MAX_D) return me_fail("me_attention_general: value head size %d must be in 1..%d", dv, AG_MAX_D);
   if (keep_first < 0 || (keep_first > 0 && window <= 0))
     return me_fail("me_attention_general: keep_first=%d needs a window", keep_first);
   if (unturn && (dv % 2 || (un_pairing & ~1))) return me_fail("me_attention_general: values of size %d, pairing %d", dv, un_pairing);
-  const bool plain = dv == d && keep_first == 0 && !unturn;
+  const bool plain = dv == d && keep_first == 0 && !unturn && !sink && !gate;
   if (nh <= 0 || nkv <= 0 || nh % nkv)
     return me_fail("me_attention_general: %d query heads are not a multiple of %d key/value heads", nh, nkv);
   if (bs <= 0 || table_width <= 0 || window < 0)
@@ -502,12 +514,24 @@ extern "C" int me_attention_general_ext(const void* q, const void* k_cache, cons
   if (dtype == ME_F32)
     attention_general_kernel<float><<<blocks, waves * 64, 0, stream>>>(
         (const float*)q, (const float*)k_cache, (const float*)v_cache, positions, token_item, block_table,
-        table_width, (float*)out, num_tokens, nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu);
+        table_width, (float*)out, num_tokens, nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu, sink,
+        (const float*)gate, (size_t)gate_row);
   else
     attention_general_kernel<bf16_t><<<blocks, waves * 64, 0, stream>>>(
         (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, token_item, block_table,
-        table_width, (bf16_t*)out, num_tokens, nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu);
+        table_width, (bf16_t*)out, num_tokens, nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu, sink,
+        (const bf16_t*)gate, (size_t)gate_row);
   return me_check_launch("me_attention_general");
+}
+
+extern "C" int me_attention_general_ext(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                                        const int* token_item, const int* block_table, int table_width, void* out,
+                                        int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
+                                        const float* unturn, int un_pairing, float scale, int dtype, int items,
+                                        hipStream_t stream) {
+  return me_attention_general_gated(q, k_cache, v_cache, positions, token_item, block_table, table_width, out, num_tokens, nh, nkv,
+                                    d, dv, bs, window, keep_first, unturn, un_pairing, scale, nullptr, nullptr, 0, dtype, items,
+                                    stream);
 }
 
 extern "C" int me_attention_general(const void* q, const void* k_cache, const void* v_cache, const int* positions,

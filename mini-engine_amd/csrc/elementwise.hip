@@ -996,13 +996,14 @@ __global__ __launch_bounds__(256) void qkv_rotate_scatter_kernel(
     const float* __restrict__ rope_table, int rd, int pairing, const float* __restrict__ v_table, int v_pairing,
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
     int table_width, T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int nkv, int d, int dv,
-    int bs, float eps, int heads_per_block, int skip_v) {
+    int bs, float eps, int heads_per_block, int skip_v, size_t width, float q_temp_coef, int q_temp_every) {
   __shared__ float stage[4][ME_MAX_HEAD_DIM];
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int t = blockIdx.x;
   const int heads_total = skip_v ? nh + nkv : nh + 2 * nkv;  // (value heads may be written by the page-tile kernel)
-  const size_t width = (size_t)(nh + nkv) * d + (size_t)nkv * dv;
   const int pos = positions[t];
+  // a temperature on the queries that grows with the position by steps: 1 + coef * ln(floor((pos + 1) / every) + 1)
+  const float q_temp = q_temp_every > 0 ? 1.f + q_temp_coef * logf((float)((pos + 1) / q_temp_every + 1)) : 1.f;
   const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
   const int hd_end = min(heads_total, (int)(blockIdx.y + 1) * heads_per_block);
   for (int hd = blockIdx.y * heads_per_block + wave; hd < hd_end; hd += 4) {
@@ -1056,7 +1057,7 @@ __global__ __launch_bounds__(256) void qkv_rotate_scatter_kernel(
 #pragma unroll
       for (int k = 0; k < ME_MAX_HEAD_DIM / ME_WAVE; ++k) {
         const int i = lane + k * ME_WAVE;
-        if (i < d) dst[i] = from_float<T>(vals[k]);
+        if (i < d) dst[i] = from_float<T>(vals[k] * q_temp);
       }
     } else if (page >= 0) {
       if (kind == 1) {
@@ -1080,13 +1081,20 @@ __global__ __launch_bounds__(256) void qkv_rotate_scatter_kernel(
 
 // item_start / num_items / num_segments: when given (num_segments > 0: the sum over items of (pos0 + qlen - 1)/16 - pos0/16
 // + 1) and the values have the keys' size, the values are turned and written a page segment of 16 slots at a time.
-extern "C" int me_qkv_rotate_scatter_tiles(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd,
-                                           int pairing, const float* v_table, int v_pairing, const int* positions,
-                                           const int* token_item, const int* block_table, int table_width, void* q_out,
-                                           void* k_cache, void* v_cache, int num_tokens, int nh, int nkv, int d, int dv, int bs,
-                                           float eps, int dtype, const int* item_start, int num_items, int num_segments,
-                                           hipStream_t stream) {
+// row_stride: elements from one token's row of qkv to the next (0: the rows hold q, k and v and nothing else; a wider row
+// carries columns behind them that this kernel does not read; the page-segment form of the values takes plain rows only).
+// q_temp_every > 0: every query is multiplied by 1 + q_temp_coef * ln(floor((position + 1) / q_temp_every) + 1).
+extern "C" int me_qkv_rotate_scatter_rows(const void* qkv, long long row_stride, const float* q_w, const float* k_w,
+                                          const float* rope_table, int rd, int pairing, const float* v_table, int v_pairing,
+                                          float q_temp_coef, int q_temp_every, const int* positions, const int* token_item,
+                                          const int* block_table, int table_width, void* q_out, void* k_cache, void* v_cache,
+                                          int num_tokens, int nh, int nkv, int d, int dv, int bs, float eps, int dtype,
+                                          const int* item_start, int num_items, int num_segments, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
+  const size_t plain_width = (size_t)(nh + nkv) * d + (size_t)nkv * dv;
+  if (row_stride != 0 && (size_t)row_stride < plain_width) return me_fail("me_qkv_rotate_scatter: rows of %lld elements are too short", row_stride);
+  const size_t width = row_stride ? (size_t)row_stride : plain_width;
+  if (width != plain_width) num_segments = 0;
   if (d <= 0 || d > ME_MAX_HEAD_DIM || dv <= 0 || dv > ME_MAX_HEAD_DIM)
     return me_fail("me_qkv_rotate_scatter: head sizes %d and %d must be in 1..%d", d, dv, ME_MAX_HEAD_DIM);
   if (rope_table && (rd <= 0 || rd > d || rd % 2)) return me_fail("me_qkv_rotate_scatter: rotary_dim=%d with head_dim=%d", rd, d);
@@ -1102,7 +1110,8 @@ extern "C" int me_qkv_rotate_scatter_tiles(const void* qkv, const float* q_w, co
   if (dtype == ME_F32) {
     qkv_rotate_scatter_kernel<float><<<grid, 256, 0, stream>>>(
         (const float*)qkv, q_w, k_w, rope_table, rd, pairing, v_table, v_pairing, positions, token_item, block_table, table_width,
-        (float*)q_out, (float*)k_cache, (float*)v_cache, nh, nkv, d, dv, bs, eps, hpb, tiles ? 1 : 0);
+        (float*)q_out, (float*)k_cache, (float*)v_cache, nh, nkv, d, dv, bs, eps, hpb, tiles ? 1 : 0, width, q_temp_coef,
+        q_temp_every);
     if (tiles)
       v_scatter_tiles_kernel<float><<<dim3(num_segments, nkv), 256, 0, stream>>>(
           (const float*)qkv, positions, item_start, num_items, block_table, table_width, (float*)v_cache, nh, nkv, d, bs, v_table,
@@ -1110,13 +1119,25 @@ extern "C" int me_qkv_rotate_scatter_tiles(const void* qkv, const float* q_w, co
   } else {
     qkv_rotate_scatter_kernel<bf16_t><<<grid, 256, 0, stream>>>(
         (const bf16_t*)qkv, q_w, k_w, rope_table, rd, pairing, v_table, v_pairing, positions, token_item, block_table, table_width,
-        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, dv, bs, eps, hpb, tiles ? 1 : 0);
+        (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, nh, nkv, d, dv, bs, eps, hpb, tiles ? 1 : 0, width, q_temp_coef,
+        q_temp_every);
     if (tiles)
       v_scatter_tiles_kernel<bf16_t><<<dim3(num_segments, nkv), 256, 0, stream>>>(
           (const bf16_t*)qkv, positions, item_start, num_items, block_table, table_width, (bf16_t*)v_cache, nh, nkv, d, bs, v_table,
           v_pairing);
   }
   return me_check_launch("me_qkv_rotate_scatter");
+}
+
+extern "C" int me_qkv_rotate_scatter_tiles(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd,
+                                           int pairing, const float* v_table, int v_pairing, const int* positions,
+                                           const int* token_item, const int* block_table, int table_width, void* q_out,
+                                           void* k_cache, void* v_cache, int num_tokens, int nh, int nkv, int d, int dv, int bs,
+                                           float eps, int dtype, const int* item_start, int num_items, int num_segments,
+                                           hipStream_t stream) {
+  return me_qkv_rotate_scatter_rows(qkv, 0, q_w, k_w, rope_table, rd, pairing, v_table, v_pairing, 0.f, 0, positions, token_item,
+                                    block_table, table_width, q_out, k_cache, v_cache, num_tokens, nh, nkv, d, dv, bs, eps, dtype,
+                                    item_start, num_items, num_segments, stream);
 }
 
 extern "C" int me_qkv_rotate_scatter(const void* qkv, const float* q_w, const float* k_w, const float* rope_table, int rd,

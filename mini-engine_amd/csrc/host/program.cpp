@@ -140,7 +140,15 @@ SplitPlan split_plan(int items, int kv_units, int max_ctx, int least_live, const
 // An attention operation that the kernels of the plain form serve: keys and values of one size, a window without kept
 // first keys, rotation of halves, values as they are.
 bool attention_is_plain(const Op& op) {
-  return (op.i[9] == 0 || op.i[9] == op.i[2]) && op.i[10] == 0 && op.i[11] == 0 && op.i[12] == 0;
+  return (op.i[9] == 0 || op.i[9] == op.i[2]) && op.i[10] == 0 && op.i[11] == 0 && op.i[12] == 0 && op.i[13] == 0 && op.i[14] == 0;
+}
+
+// How many residual streams the tokens of a program have (kOpStreams; 1 without).
+int streams_of(const std::vector<Op>& ops) {
+  int s = 1;
+  for (const Op& op : ops)
+    if (op.kind == kOpStreams) s = std::max(s, (int)op.i[0]);
+  return s;
 }
 
 // Whether prompts of an attention operation beyond the plain form go to the tiled matrix-core kernel: bfloat16, keys and
@@ -158,8 +166,8 @@ class Run {
   Run(const Program& prog, const std::vector<Value>& values, const StepView& s, Arena& arena, int32_t* fed_tokens,
       hipStream_t stream)
       : prog_(prog), values_(values), s_(s), arena_(arena), fed_tokens_(fed_tokens), stream_(stream), dtype_(prog.dtype()),
-        elem_(prog.dtype() == kF32 ? 4 : 2), t_(s.lay.tokens), h_(prog.hidden()) {
-    x_ = (float*)arena_.take((size_t)t_ * h_ * 4);
+        elem_(prog.dtype() == kF32 ? 4 : 2), t_(s.lay.tokens), h_(prog.hidden()), streams_(streams_of(prog.ops())) {
+    x_ = (float*)arena_.take((size_t)streams_ * t_ * h_ * 4);  // (several streams: [streams, tokens, hidden], x_ is the first)
     spare_ = (float*)arena_.take((size_t)t_ * h_ * 4);
     normed_ = arena_.take((size_t)t_ * h_ * elem_);
     for (const Value& v : values) bufs_.push_back(arena_.take((size_t)t_ * v.cols * v.elem));
@@ -177,7 +185,7 @@ class Run {
       step(op);
       // the logits, the drawn tokens and partial sums that wait for the next norm outlive their operation;
       // an operation that used up waiting partial sums gives their memory back too
-      if (op.kind != kOpHead && op.kind != kOpHeadRows && op.kind != kOpSample && op.kind != kOpLinearDelta)
+      if (op.kind != kOpHead && op.kind != kOpHeadRows && op.kind != kOpStreamHead && op.kind != kOpSample && op.kind != kOpLinearDelta)
         arena_.used = released_to_ != (size_t)-1 ? released_to_ : mark;
     }
     return result_;
@@ -250,6 +258,23 @@ class Run {
         break;
       case kOpHeadRows:
         head_rows(op);
+        break;
+      case kOpStreams:
+        if (pending_.any() || held_.any() || pending_.carried()) throw Error(kBroken, "a result is pending where the streams begin");
+        ok(me_streams_spread(x_, (long long)t_ * h_, streams_, stream_));
+        spread_ = true;
+        break;
+      case kOpStreamNorm:
+        stream_norm(op, bufs_[op.out], nullptr, t_, 1);
+        break;
+      case kOpStreamHead:
+        stream_head(op);
+        break;
+      case kOpLatentAttention:
+        latent_attention(op);
+        break;
+      case kOpRoutedFF:
+        routed_ff(op);
         break;
       default:
         throw Error(kBadValue, "unknown operation in a step program");
@@ -382,6 +407,7 @@ class Run {
     if (n != h_) throw Error(kBadValue, "a delta of the residual stream has the hidden size");
     const void* x = bufs_[op.in];
     const float scale = scale_of(op.f[0]);
+    const bool stays = op.i[2] != 0 || spread_;  // the result waits for whatever rewrites the stream(s) behind it
     pending_ = Pending();
     pending_.scale = scale;
     if (attn_parts_.o) {  // decode attention left its splits to this product
@@ -397,7 +423,7 @@ class Run {
       pending_.stride = (long long)t_ * n;
       return;
     }
-    if (scale == 1.f && !held_.any() && next_ && next_->kind == kOpNormLinear && next_->i[1] == h_ && groups_of(next_->i[3]) == 1 &&
+    if (!stays && scale == 1.f && !held_.any() && next_ && next_->kind == kOpNormLinear && next_->i[1] == h_ && groups_of(next_->i[3]) == 1 &&
         choose_carried_norm(dtype_, t_, n, k, (int)next_->i[0], (int)next_->i[2], compute_units(), true)) {
       // x += product in the product's epilogue, which also starts the norm behind it (choice.cpp)
       const int blocks = me_gemm_bf16_stream_carry_blocks(t_, n, k, compute_units());
@@ -411,7 +437,7 @@ class Run {
     }
     const ProductChoice c = choose_product(dtype_, kRoleDeltaInto, t_, n, k, 0, dtype_, compute_units(), true);
     if (c.adds_into) {  // x += product, in the library's epilogue: nothing stays pending
-      if (scale == 1.f && library_adds(x, op.p[1], x_, t_, n, k, stream_)) {  // (a result set aside waits for the next add as before)
+      if (!stays && scale == 1.f && library_adds(x, op.p[1], x_, t_, n, k, stream_)) {  // (a result set aside waits for the next add as before)
         pending_ = Pending();
         return;
       }
@@ -462,12 +488,15 @@ class Run {
       const int v_pairing = op.i[12] ? (int)op.i[12] - 1 : 0;
       if (!owns) throw Error(kBadValue, "an attention layer of this form writes its own pages");
       void* q = arena_.take((size_t)t_ * nh * d * elem_);
+      const bool gated = op.i[14] != 0;  // the rows end in a gate per head
+      const long long row = (long long)(nh + nkv) * d + (long long)nkv * dv + (gated ? nh : 0);
+      const char* gate = gated ? (const char*)qkv + (size_t)(row - nh) * elem_ : nullptr;
       int segments = 0;
-      if (t_ >= 64 && dv == d)  // many tokens: the values are turned and written a page segment (a transposed tile) at a time
+      if (t_ >= 64 && dv == d && !gated)  // many tokens: the values are turned and written a page segment (a transposed tile) at a time
         for (int i = 0; i < items; ++i) segments += (s_.starts[i] + s_.qlens[i] - 1) / 16 - s_.starts[i] / 16 + 1;
-      ok(me_qkv_rotate_scatter_tiles(qkv, q_w, k_w, rope, rd, pairing, v_table, v_pairing, idx(s_.lay.positions),
-                                     idx(s_.lay.token_item), table, width, q, kc, vc, t_, nh, nkv, d, dv, bs, eps, dtype_,
-                                     segments ? idx(s_.lay.item_start) : nullptr, items, segments, stream_));
+      ok(me_qkv_rotate_scatter_rows(qkv, gated ? row : 0, q_w, k_w, rope, rd, pairing, v_table, v_pairing, op.f[2], (int)op.i[13],
+                                    idx(s_.lay.positions), idx(s_.lay.token_item), table, width, q, kc, vc, t_, nh, nkv, d, dv, bs, eps,
+                                    dtype_, segments ? idx(s_.lay.item_start) : nullptr, items, segments, stream_));
       if (s_.decode_only && attention_takes_tiled_prefill(op, dtype_)) {
         // one new token per item: the split-context kernel, which deals the kept first keys' tiles to its splits before
         // the window's; a second kernel (or the blocks themselves) adds up the splits
@@ -479,6 +508,7 @@ class Run {
                                          window, keep_first, scale, sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits,
                                          kDecodeWaves, idx(s_.lay.live_items) + 1, stream_));
         if (v_table) ok(me_unturn_rows(out, v_table, v_pairing, idx(s_.lay.positions), t_, nh, dv, dtype_, stream_));
+        if (gate) ok(me_head_gate(out, gate, row, t_, nh, dv, dtype_, stream_));
         return;
       }
       if (!s_.decode_only && attention_takes_tiled_prefill(op, dtype_)) {
@@ -496,10 +526,11 @@ class Run {
                                           part_ml, p.token_chunks >= 0 ? idx(p.token_chunks) : nullptr, p.max_chunks, t_, nh, nkv, d,
                                           bs, window, keep_first, scale, p.columns, stream_));
         if (v_table) ok(me_unturn_rows(out, v_table, v_pairing, idx(s_.lay.positions), t_, nh, dv, dtype_, stream_));
+        if (gate) ok(me_head_gate(out, gate, row, t_, nh, dv, dtype_, stream_));
         return;
       }
-      ok(me_attention_general_ext(q, kc, vc, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, out, t_, nh, nkv, d, dv, bs,
-                                  window, keep_first, v_table, v_pairing, scale, dtype_, items, stream_));
+      ok(me_attention_general_gated(q, kc, vc, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, out, t_, nh, nkv, d, dv,
+                                    bs, window, keep_first, v_table, v_pairing, scale, nullptr, gate, row, dtype_, items, stream_));
       return;
     }
     const bool mfma = dtype_ == kBF16 && me_attention_mfma_supported(d, bs) && group <= 16;
@@ -593,6 +624,76 @@ class Run {
                       d, dv, (int)op.i[5], op.f[0], (int)op.i[6], (int)op.i[7], op.f[1], dtype_, longest, stream_));
   }
 
+  // The pending result rewrites the streams (by the coefficients of the part that gave it), the coming part's input is
+  // read from them and normed: one kernel.
+  void stream_norm(const Op& op, void* out, const int* rows, int num_rows, int write_x) {
+    if (!spread_) throw Error(kBroken, "a norm over several streams before the streams begin");
+    if (held_.any() || pending_.carried()) throw Error(kBroken, "several streams take one pending result at a time");
+    if (pending_.any() && !op.p[op.kind == kOpStreamHead ? 2 : 1])
+      throw Error(kBroken, "a result is pending and nothing says how it rewrites the streams");
+    if (pending_.any() && pending_.scale != 1.f) throw Error(kBroken, "a result of several streams is not scaled");
+    const float* mix_out = pending_.any() ? (const float*)op.p[op.kind == kOpStreamHead ? 2 : 1] : nullptr;
+    const float* w_in = op.kind == kOpStreamHead ? nullptr : (const float*)op.p[2];
+    ok(me_streams_norm(x_, (long long)t_ * h_, streams_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride, mix_out,
+                       w_in, (const float*)op.p[0], out, rows, num_rows, h_, op.f[0], write_x, dtype_, stream_));
+    pending_ = Pending();
+    if (op.kind != kOpStreamHead) release_parts();  // (the head's buffers lie behind waiting partial sums)
+  }
+
+  void stream_head(const Op& op) {
+    const int rows = s_.lay.rows;
+    result_.rows = rows;
+    if (rows == 0) {
+      pending_ = Pending();
+      return;
+    }
+    void* picked = arena_.take((size_t)rows * h_ * elem_);
+    stream_norm(op, picked, idx(s_.lay.want_rows), rows, 0);
+    logits_of(picked, op);
+  }
+
+  // Attention over one cached latent per token (csrc/latent_attention.hip): the latent's norm, the rotation and the page
+  // write; the keys' map folded into the queries; attention over one key/value head whose values are the latents; the
+  // values' map on the weighted latents, with the output gate.
+  void latent_attention(const Op& op) {
+    const int nh = (int)op.i[0], d = (int)op.i[1], r = (int)op.i[2], rank = (int)op.i[3], dv = (int)op.i[4], bs = (int)op.i[5];
+    const int g = (int)op.i[6], dk = rank + r;
+    if (g < 0 || g >= (int)s_.lay.widths.size()) throw Error(kBadValue, "an attention layer names a cache group the step lacks");
+    if (op.i[7] < s_.max_ctx)
+      throw Error(kBadValue, "the rotary table covers " + std::to_string(op.i[7]) + " positions, the step may reach " +
+                                 std::to_string(s_.max_ctx));
+    const long long row = (long long)nh * (d + r) + dk + nh;
+    if (values_[op.in].cols != row) throw Error(kBadValue, "the projections of a latent attention layer have the wrong width");
+    const int32_t* table = idx(s_.lay.tables[g]);
+    const int width = s_.lay.widths[g];
+    const char* proj = (const char*)bufs_[op.in];
+    void* qa = arena_.take((size_t)t_ * nh * dk * elem_);
+    void* ol = arena_.take((size_t)t_ * nh * rank * elem_);
+    ok(me_latent_prepare(proj, row, (const float*)op.p[0], (const float*)op.p[1], idx(s_.lay.positions), idx(s_.lay.token_item), table,
+                         width, qa, (void*)op.p[2], (void*)op.p[3], t_, nh, d, r, rank, rank, bs, op.f[0], dtype_, stream_));
+    ok(me_head_product(proj, row, d + r, op.p[4], qa, (long long)nh * dk, dk, nullptr, 0, t_, nh, rank, d, dtype_, stream_));
+    ok(me_attention_general_gated(qa, op.p[2], op.p[3], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, ol, t_, nh, 1, dk,
+                                  rank, bs, 0, 0, nullptr, 0, op.f[1], (const float*)op.p[6], nullptr, 0, dtype_, s_.lay.items,
+                                  stream_));
+    ok(me_head_product(ol, (long long)nh * rank, rank, op.p[5], bufs_[op.out], (long long)nh * dv, dv,
+                       proj + (size_t)(row - nh) * elem_, row, t_, nh, dv, rank, dtype_, stream_));
+  }
+
+  // A feed-forward of routed experts (csrc/routed_ff.hip): its result waits as one partial sum per expert of a token.
+  void routed_ff(const Op& op) {
+    const int E = (int)op.i[0], top = (int)op.i[1], ff = (int)op.i[2];
+    pending_ = Pending();
+    parts_mark_ = arena_.used;
+    float* parts = (float*)arena_.take((size_t)top * t_ * h_ * 4);
+    released_to_ = arena_.used;  // the partial sums outlive this operation, its workspace does not
+    void* ws = arena_.take((size_t)me_routed_ff_workspace(t_, E, top, ff, elem_));
+    ok(me_routed_ff(bufs_[op.in], (const float*)op.p[0], op.p[1], op.p[2], parts, ws, t_, h_, E, top, ff, (int)op.i[3], dtype_,
+                    stream_));
+    pending_.parts = parts;
+    pending_.num_parts = top;
+    pending_.stride = (long long)t_ * h_;
+  }
+
   // Rows are selected before the final norm, as the reference does (model.py:186); logits are float32.
   void head(const Op& op) {
     const int rows = s_.lay.rows;
@@ -665,7 +766,8 @@ class Run {
   Arena& arena_;
   int32_t* fed_tokens_;
   hipStream_t stream_;
-  const int dtype_, elem_, t_, h_;
+  const int dtype_, elem_, t_, h_, streams_;
+  bool spread_ = false;  // the streams are in use (kOpStreams has run)
   float *x_, *spare_;
   void* normed_;
   std::vector<void*> bufs_;
@@ -706,7 +808,7 @@ std::vector<std::vector<int>> Program::prefill_geometries() const {
 size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t max_ctx) const {
   const size_t elem = dtype_ == kF32 ? 4 : 2;
   const size_t pad = 256;
-  size_t fixed = 2 * ((size_t)tokens * hidden_ * 4 + pad) + (size_t)tokens * hidden_ * elem + pad;
+  size_t fixed = (1 + (size_t)streams_of(ops_)) * ((size_t)tokens * hidden_ * 4 + pad) + (size_t)tokens * hidden_ * elem + pad;
   for (const Value& v : values_) fixed += (size_t)tokens * v.cols * v.elem + pad;
   size_t scratch = 0;
   for (const Op& op : ops_) {
@@ -716,6 +818,11 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
       need = std::max<size_t>((size_t)kMaxRuns * std::min<int64_t>(tokens, kSmallMaxRows), (size_t)tokens) * op.i[0] * 4 + pad;
     if (op.kind == kOpDecayState)
       need = (size_t)me_decay_state_workspace(tokens, items, (int)op.i[0], (int)op.i[1], (int)op.i[2]) + pad;
+    if (op.kind == kOpLatentAttention)
+      need = (size_t)tokens * op.i[0] * (2 * op.i[3] + op.i[2]) * elem + 2 * pad;
+    if (op.kind == kOpRoutedFF)
+      need = (size_t)op.i[1] * tokens * hidden_ * 4 + (size_t)me_routed_ff_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2], (int)elem) +
+             2 * pad;
     if (op.kind == kOpAttention && !attention_is_plain(op)) {
       need = (size_t)tokens * op.i[0] * op.i[2] * elem + pad;
       if (attention_takes_tiled_prefill(op, dtype_)) {  // the splits' partial results of a decode step

@@ -50,7 +50,27 @@ enum OpKind {
                       // -> out [tokens, heads * dv]
   kOpHold = 13,       // the pending delta is set aside until the next add: a second part that reads the same normed input
                       // follows, and the add takes both results at once (with the same multiplier)
+  kOpStreams = 14,    // i0 S: from here on a token has S residual streams [S, tokens, hidden], each a copy of x as it is now
+  kOpStreamNorm = 15, // p0 norm weight, f0 eps, p1 float32 [S * S + S]: how the pending result rewrites the streams (mix[from, to],
+                      // then out[to]; null: nothing is pending), p2 float32 [S]: what the coming part reads of each stream;
+                      // pending + streams -> streams, out [tokens, hidden]
+  kOpStreamHead = 16, // p0 final norm weight, f0 eps, p1 head W, f1 the scale on the logits, p2 as p1 of kOpStreamNorm: the sum of the
+                      // streams of the wanted rows, normed -> logits
+  kOpLatentAttention = 17,  // in: projections [tokens, heads (d + r) | rank + r | heads] (queries, the latent and the shared rotated
+                      // key part, a gate per head); p0 weight of the latent's norm, p1 rotary table [positions, 2, r/2], p2 key
+                      // pages [page, 1, slot, rank + r], p3 value pages [page, 1, rank, slot], p4 the keys' map per head, transposed
+                      // [heads, rank, d], p5 the values' map per head [heads, dv, rank], p6 sink float32 [heads] or null;
+                      // i0 heads, i1 d, i2 r, i3 rank, i4 dv, i5 page size, i6 cache group, i7 positions the table covers;
+                      // f0 eps, f1 scale -> out [tokens, heads * dv]
+  kOpRoutedFF = 18,   // in: normed activations; p0 router W float32 [E, hidden], p1 experts' gate and up rows [E, 2 ff, hidden],
+                      // p2 experts' down rows [E, hidden, ff]; i0 E, i1 experts a token, i2 ff, i3 code of the activation
+                      // -> pending (partial sums, one per expert of a token)
 };
+// kOpLinearDelta i2: the result stays pending whatever the step's size (no product adds itself to the stream).
+// kOpAttention beyond i12: i13 every (0: none) and f2 coef of a temperature on the queries, 1 + coef * ln(floor((position + 1) / every)
+// + 1); i14: the input ends in one more column per head, a gate whose sigmoid multiplies the head's output.
+
+constexpr int kOpPtrs = 8;
 
 constexpr int kOpInts = 16, kOpFloats = 4;
 
@@ -69,7 +89,7 @@ typedef int (*CallFn)(const CallFrame*);
 
 struct Op {
   int kind = 0, in = -1, out = -1;
-  const void* p[6] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+  const void* p[kOpPtrs] = {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
   int64_t i[kOpInts] = {0};
   float f[kOpFloats] = {0.f, 0.f, 0.f, 0.f};
 };

@@ -117,10 +117,10 @@ int me_runner_value(void* runner, int64_t cols, int elem) {
                return ((Runner*)runner)->prog.add_value(cols, elem);)
 }
 
-// ptrs: 6 pointers, ints: 10, floats: 2 (see OpKind in program.h for what each operation reads).
+// ptrs: kOpPtrs pointers, ints: kOpInts, floats: kOpFloats (see OpKind in program.h for what each operation reads).
 int me_runner_op(void* runner, int kind, int in, int out, const void* const* ptrs, const int64_t* ints, const float* floats) {
   ME_RUN_GUARD(me::Op op; op.kind = kind; op.in = in; op.out = out;
-               for (int i = 0; i < 6; ++i) op.p[i] = ptrs[i];
+               for (int i = 0; i < me::kOpPtrs; ++i) op.p[i] = ptrs[i];
                for (int i = 0; i < me::kOpInts; ++i) op.i[i] = ints[i];
                for (int i = 0; i < me::kOpFloats; ++i) op.f[i] = floats[i];
                Runner* r = (Runner*)runner; r->prog.add_op(op); r->geometries = r->prog.prefill_geometries();

@@ -90,6 +90,31 @@ int me_attention_decode_bf16_kept(const void* q, const void* k_cache, const void
                                   int nh, int nkv, int d, int bs, int window, int keep_first, float scale, int split_keys,
                                   int num_splits, int max_ctx, const int* live_items, int full_splits, int waves_wanted,
                                   const int* step_flags, hipStream_t stream);
+int me_attention_general_gated(const void* q, const void* k_cache, const void* v_cache, const int* positions,
+                               const int* token_item, const int* block_table, int table_width, void* out, int num_tokens, int nh,
+                               int nkv, int d, int dv, int bs, int window, int keep_first, const float* unturn, int un_pairing,
+                               float scale, const float* sink, const void* gate, long long gate_row, int dtype, int items,
+                               hipStream_t stream);
+int me_qkv_rotate_scatter_rows(const void* qkv, long long row_stride, const float* q_w, const float* k_w, const float* rope_table,
+                               int rd, int pairing, const float* v_table, int v_pairing, float q_temp_coef, int q_temp_every,
+                               const int* positions, const int* token_item, const int* block_table, int table_width, void* q_out,
+                               void* k_cache, void* v_cache, int num_tokens, int nh, int nkv, int d, int dv, int bs, float eps,
+                               int dtype, const int* item_start, int num_items, int num_segments, hipStream_t stream);
+int me_streams_spread(float* xs, long long per_stream, int S, hipStream_t stream);
+int me_streams_norm(float* xs, long long per_stream, int S, const void* delta, const float* parts, int num_parts,
+                    long long part_stride, const float* mix_out, const float* w_in, const float* w, void* h, const int* rows,
+                    int num_rows, int dim, float eps, int write_x, int dtype, hipStream_t stream);
+int me_latent_prepare(const void* proj, long long row_stride, const float* norm_w, const float* rope, const int* positions,
+                      const int* token_item, const int* block_table, int table_width, void* qa, void* k_cache, void* v_cache,
+                      int num_tokens, int nh, int d, int r, int rank, int v_rows, int bs, float eps, int dtype, hipStream_t stream);
+int me_head_product(const void* x, long long x_row, long long x_head, const void* W, void* out, long long out_row,
+                    long long out_head, const void* gate, long long gate_row, int num_tokens, int heads, int n, int k, int dtype,
+                    hipStream_t stream);
+int me_head_gate(void* rows, const void* gate, long long gate_row, int num_tokens, int heads, int n, int dtype, hipStream_t stream);
+int me_routed_ff_max_tiles(long long tokens, int E, int top);
+long long me_routed_ff_workspace(long long tokens, int E, int top, int ff, int elem);
+int me_routed_ff(const void* h, const float* Wr, const void* W_gu, const void* W_down, float* parts, void* workspace, int num_tokens,
+                 int hidden, int E, int top, int ff, int act, int dtype, hipStream_t stream);
 int me_unturn_rows(void* rows, const float* table, int pairing, const int* positions, int num_tokens, int heads, int n,
                    int dtype, hipStream_t stream);
 int me_gemm_f32(const float* A, const float* W, float* C, int M, int N, int K, hipStream_t stream);

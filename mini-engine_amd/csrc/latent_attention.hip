@@ -1,0 +1,152 @@
+// Attention over one latent per token (keys and values of all heads are linear maps of it), in the form that never
+// expands the latents: with c the normed latent [rank] and k_r the rotated key part [r] that all heads share,
+//   score_h(i, j) = q_h[:d] . (W_uk_h c_j) + rot(q_h[d:]) . k_r_j = (W_uk_h^T q_h[:d]) . c_j + rot(q_h[d:]) . k_r_j
+//   out_h(i)      = W_uv_h (sum_j p_h(i, j) c_j)
+// so a layer caches one key [c | k_r] per token (one key/value head for all query heads) whose first `rank` elements
+// are also its value. The kernels here prepare that: the latent's norm, the rotation, the page write, and the two small
+// products per head (W_uk_h^T on the queries, W_uv_h on the weighted latents, with the output gate). The attention
+// itself is the framework's, over a page pool with one key/value head.
+#include "tile_product.h"
+
+// proj [T, row_stride]: nh query heads of (d + r), then rank + r elements of the latent projection (what follows in the
+// row is not read here). One block per token:
+//   c = latent[:rank] * rsqrt(mean(latent[:rank]^2) + eps) * norm_w  -> K[page, 0, slot, :rank], V[page, 0, :rank, slot]
+//   k_r = latent[rank:] turned by the position's angles (element i with i + r/2)  -> K[page, 0, slot, rank:]
+//   (with value rows for the whole key, v_rows == rank + r, also V[page, 0, rank:, slot])
+//   every head's q[d:] turned likewise -> qa[t, h, rank:]   (qa [T, nh, rank + r]; its first rank elements are the
+//   product of the kernel below)
+// rope: float32 [positions, 2, r/2], cosines then sines, already multiplied by whatever the encoding multiplies them by.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prepare_kernel(
+    const T* __restrict__ proj, size_t row_stride, const float* __restrict__ norm_w, const float* __restrict__ rope,
+    const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table, int table_width,
+    T* __restrict__ qa, T* __restrict__ k_cache, T* __restrict__ v_cache, int nh, int d, int r, int rank, int v_rows, int bs,
+    float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, dk = rank + r, half = r / 2;
+  const int pos = positions[t];
+  const int page = block_table[(size_t)token_item[t] * table_width + pos / bs], slot = pos % bs;
+  const T* row = proj + (size_t)t * row_stride;
+  const T* lat = row + (size_t)nh * (d + r);
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+    const float v = to_float(lat[i]);
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = rsqrtf(block_sum(ss, scratch) / (float)rank + eps);
+  const float* cs = rope + (size_t)pos * r;
+  if (page >= 0) {
+    T* krow = k_cache + ((size_t)page * bs + slot) * dk;
+    T* vcol = v_cache + (size_t)page * v_rows * bs + slot;
+    for (int i = threadIdx.x; i < rank; i += blockDim.x) {
+      const T c = from_float<T>(to_float(lat[i]) * inv * norm_w[i]);
+      krow[i] = c;
+      vcol[(size_t)i * bs] = c;
+    }
+    for (int i = threadIdx.x; i < r; i += blockDim.x) {
+      const bool first = i < half;
+      const int j = first ? i : i - half;
+      const float a = to_float(lat[rank + i]), b = to_float(lat[rank + (first ? i + half : i - half)]);
+      const T v = from_float<T>(first ? a * cs[j] - b * cs[half + j] : a * cs[j] + b * cs[half + j]);
+      krow[rank + i] = v;
+      if (v_rows == dk) vcol[(size_t)(rank + i) * bs] = v;
+    }
+  }
+  for (int idx = threadIdx.x; idx < nh * r; idx += blockDim.x) {
+    const int h = idx / r, i = idx % r;
+    const T* src = row + (size_t)h * (d + r) + d;
+    const bool first = i < half;
+    const int j = first ? i : i - half;
+    const float a = to_float(src[i]), b = to_float(src[first ? i + half : i - half]);
+    qa[((size_t)t * nh + h) * dk + rank + i] = from_float<T>(first ? a * cs[j] - b * cs[half + j] : a * cs[j] + b * cs[half + j]);
+  }
+}
+
+extern "C" int me_latent_prepare(const void* proj, long long row_stride, const float* norm_w, const float* rope,
+                                 const int* positions, const int* token_item, const int* block_table, int table_width, void* qa,
+                                 void* k_cache, void* v_cache, int num_tokens, int nh, int d, int r, int rank, int v_rows, int bs,
+                                 float eps, int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (nh <= 0 || d <= 0 || rank <= 0 || r <= 0 || r % 2) return me_fail("me_latent_prepare: heads=%d d=%d rank=%d rot=%d", nh, d, rank, r);
+  if (v_rows != rank && v_rows != rank + r) return me_fail("me_latent_prepare: value pages of %d rows for a latent of %d + %d", v_rows, rank, r);
+  if (row_stride < (long long)nh * (d + r) + rank + r) return me_fail("me_latent_prepare: rows of %lld elements are too short", row_stride);
+  if (bs <= 0 || table_width <= 0) return me_fail("me_latent_prepare: block_size=%d table_width=%d", bs, table_width);
+  if (dtype == ME_F32)
+    latent_prepare_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)proj, (size_t)row_stride, norm_w, rope, positions,
+                                                                 token_item, block_table, table_width, (float*)qa, (float*)k_cache,
+                                                                 (float*)v_cache, nh, d, r, rank, v_rows, bs, eps);
+  else
+    latent_prepare_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)proj, (size_t)row_stride, norm_w, rope, positions,
+                                                                  token_item, block_table, table_width, (bf16_t*)qa,
+                                                                  (bf16_t*)k_cache, (bf16_t*)v_cache, nh, d, r, rank, v_rows, bs, eps);
+  return me_check_launch("me_latent_prepare");
+}
+
+// A product per head: out[t, h, j] = sum_i x[t, h, i] W[h, j, i] for j < n, i < k, times sigmoid(gate[t, h]) if a gate is
+// given. x, out and gate are addressed by strides in elements (row = token, head), so they may be slices of wider rows.
+// Grid (tiles of 16 tokens, tiles of 64 columns, heads).
+template <typename T>
+__global__ __launch_bounds__(256) void head_product_kernel(const T* __restrict__ x, size_t x_row, size_t x_head,
+                                                           const T* __restrict__ W, T* __restrict__ out, size_t out_row,
+                                                           size_t out_head, const T* __restrict__ gate, size_t gate_row,
+                                                           int num_tokens, int n, int k) {
+  __shared__ TileLds lds;
+  const int t0 = blockIdx.x * TP_ROWS, c0 = blockIdx.y * TP_COLS, h = blockIdx.z;
+  const int rows = min(TP_ROWS, num_tokens - t0), cols = min(TP_COLS, n - c0);
+  float acc[4];
+  tile_product<T>([&](int i) { return x + (size_t)(t0 + i) * x_row + (size_t)h * x_head; }, rows, W + ((size_t)h * n + c0) * k,
+                  cols, k, acc, lds);
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  if (tx >= cols) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = ty + 4 * i;
+    if (row < rows) {
+      float v = acc[i];
+      if (gate) v *= 1.f / (1.f + expf(-to_float(gate[(size_t)(t0 + row) * gate_row + h])));
+      out[(size_t)(t0 + row) * out_row + (size_t)h * out_head + c0 + tx] = from_float<T>(v);
+    }
+  }
+}
+
+extern "C" int me_head_product(const void* x, long long x_row, long long x_head, const void* W, void* out, long long out_row,
+                               long long out_head, const void* gate, long long gate_row, int num_tokens, int heads, int n, int k,
+                               int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads <= 0 || heads > 65535 || n <= 0 || k <= 0) return me_fail("me_head_product: heads=%d n=%d k=%d", heads, n, k);
+  const dim3 grid((num_tokens + TP_ROWS - 1) / TP_ROWS, (n + TP_COLS - 1) / TP_COLS, heads);
+  if (grid.y > 65535) return me_fail("me_head_product: %d columns a head", n);
+  if (dtype == ME_F32)
+    head_product_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, (size_t)x_row, (size_t)x_head, (const float*)W, (float*)out,
+                                                         (size_t)out_row, (size_t)out_head, (const float*)gate, (size_t)gate_row,
+                                                         num_tokens, n, k);
+  else
+    head_product_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, (size_t)x_row, (size_t)x_head, (const bf16_t*)W,
+                                                          (bf16_t*)out, (size_t)out_row, (size_t)out_head, (const bf16_t*)gate,
+                                                          (size_t)gate_row, num_tokens, n, k);
+  return me_check_launch("me_head_product");
+}
+
+// rows [T, heads, n] in place: head h of token t times sigmoid(gate[t, h]) (gate addressed by its row stride).
+template <typename T>
+__global__ void head_gate_kernel(T* __restrict__ rows, const T* __restrict__ gate, size_t gate_row, int heads, int n, size_t total) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const size_t unit = i / n;
+  const size_t t = unit / heads, h = unit % heads;
+  const float g = 1.f / (1.f + expf(-to_float(gate[t * gate_row + h])));
+  rows[i] = from_float<T>(to_float(rows[i]) * g);
+}
+
+extern "C" int me_head_gate(void* rows, const void* gate, long long gate_row, int num_tokens, int heads, int n, int dtype,
+                            hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads <= 0 || n <= 0) return me_fail("me_head_gate: heads=%d n=%d", heads, n);
+  const size_t total = (size_t)num_tokens * heads * n;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  if (dtype == ME_F32)
+    head_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)rows, (const float*)gate, (size_t)gate_row, heads, n, total);
+  else
+    head_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)rows, (const bf16_t*)gate, (size_t)gate_row, heads, n, total);
+  return me_check_launch("me_head_gate");
+}

@@ -1,0 +1,181 @@
+// A feed-forward of routed experts: a router picks `top` of E small gated feed-forwards per token and weights them by
+// the softmax over the picked logits; the token's result is the weighted sum of what they give.
+//
+//   route    z = W_r h in float32 (W_r float32), the `top` largest by repeated maximum (the lower index among equals), their
+//            weights exp(z_j - z_max) / sum; a (token, rank j) is a *pair*;
+//   sort     the pairs grouped by expert (a counting sort in one block), and a list of tiles of up to 16 pairs of one expert;
+//   gate/up  per tile: act(W_gate_e h) * (W_up_e h) for the tile's tokens -> acts [pair position, ff];
+//   down     per tile: weight * (W_down_e acts) -> parts [j, token, :] in float32: the `top` results of a token lie a
+//            stride apart, as partial sums that the next add of the residual stream sums up in the order of j.
+// A pair's result does not depend on the tile it falls into (tile_product.h), so a token's result does not depend on
+// what else the step holds. Everything stays on the device: a step that a graph replays routes anew every time.
+#include "tile_product.h"
+
+#define RF_MAX_EXPERTS 1024
+#define RF_MAX_TOP 32
+
+template <typename T>
+__global__ __launch_bounds__(256) void routed_route_kernel(const T* __restrict__ h, const float* __restrict__ Wr, int* __restrict__ ids,
+                                                           float* __restrict__ wts, int hidden, int E, int top) {
+  __shared__ float z[RF_MAX_EXPERTS];
+  const int t = blockIdx.x, wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
+  const T* row = h + (size_t)t * hidden;
+  for (int e = wave; e < E; e += 4) {
+    const float* w = Wr + (size_t)e * hidden;
+    float s = 0.f;
+    for (int c = lane; c < hidden; c += ME_WAVE) s = fmaf(to_float(row[c]), w[c], s);
+    s = wave_sum(s);
+    if (lane == 0) z[e] = s;
+  }
+  __syncthreads();
+  if (wave != 0) return;
+  float mine = 0.f, zmax = 0.f, sum = 0.f;  // lane j keeps the weight of the j-th pick
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += ME_WAVE)
+      if (z[e] > best) best = z[e], at = e;  // (ascending e: the lowest index among a lane's equals)
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, ME_WAVE);
+      const int oa = __shfl_xor(at, off, ME_WAVE);
+      if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
+    }
+    if (at >= E) at = 0;  // (a row of NaNs, as rows that pad a replayed step may be: any expert)
+    if (j == 0) zmax = best;
+    const float p = expf(best - zmax);
+    if (lane == j) mine = p;
+    sum += p;
+    if (lane == 0) {
+      ids[(size_t)t * top + j] = at;
+      z[at] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+  }
+  if (lane < top) wts[(size_t)t * top + lane] = mine / sum;
+}
+
+// plan: [0] number of tiles; [1 + 3 i ..] tile i: expert, first position, pairs; sorted [P]: the pair at each position.
+__global__ __launch_bounds__(1024) void routed_sort_kernel(const int* __restrict__ ids, int P, int E, int max_tiles,
+                                                           int* __restrict__ plan, int* __restrict__ sorted) {
+  __shared__ int count[RF_MAX_EXPERTS], first[RF_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) atomicAdd(&count[ids[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tiles = 0;
+    for (int e = 0; e < E; ++e) {
+      first[e] = at;
+      for (int b = 0; b < count[e] && tiles < max_tiles; b += TP_ROWS, ++tiles) {
+        plan[1 + 3 * tiles] = e;
+        plan[2 + 3 * tiles] = at + b;
+        plan[3 + 3 * tiles] = min(TP_ROWS, count[e] - b);
+      }
+      at += count[e];
+    }
+    plan[0] = tiles;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = first[e];
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) sorted[atomicAdd(&count[ids[p]], 1)] = p;
+}
+
+// Grid (tiles, tiles of 64 columns of ff). W_gu [E, 2 ff, hidden]: an expert's gate rows, then its up rows.
+template <typename T>
+__global__ __launch_bounds__(256) void routed_gate_up_kernel(const T* __restrict__ h, const T* __restrict__ W_gu,
+                                                             const int* __restrict__ plan, const int* __restrict__ sorted,
+                                                             T* __restrict__ acts, int hidden, int ff, int top, int act) {
+  __shared__ TileLds lds;
+  const int tile = blockIdx.x;
+  if (tile >= plan[0]) return;
+  const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
+  const int c0 = blockIdx.y * TP_COLS, cols = min(TP_COLS, ff - c0);
+  auto row_ptr = [&](int i) { return h + (size_t)(sorted[begin + i] / top) * hidden; };
+  const T* Wg = W_gu + ((size_t)e * 2 * ff + c0) * hidden;
+  float g[4], u[4];
+  tile_product<T>(row_ptr, rows, Wg, cols, hidden, g, lds);
+  tile_product<T>(row_ptr, rows, Wg + (size_t)ff * hidden, cols, hidden, u, lds);
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  if (tx >= cols) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = ty + 4 * i;
+    if (row < rows) acts[(size_t)(begin + row) * ff + c0 + tx] = from_float<T>(gate_act(g[i], act) * u[i]);
+  }
+}
+
+// Grid (tiles, tiles of 64 columns of hidden). W_down [E, hidden, ff]. parts float32 [top, tokens, hidden].
+template <typename T>
+__global__ __launch_bounds__(256) void routed_down_kernel(const T* __restrict__ acts, const T* __restrict__ W_down,
+                                                          const int* __restrict__ plan, const int* __restrict__ sorted,
+                                                          const float* __restrict__ wts, float* __restrict__ parts, int num_tokens,
+                                                          int hidden, int ff, int top) {
+  __shared__ TileLds lds;
+  const int tile = blockIdx.x;
+  if (tile >= plan[0]) return;
+  const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
+  const int c0 = blockIdx.y * TP_COLS, cols = min(TP_COLS, hidden - c0);
+  float acc[4];
+  tile_product<T>([&](int i) { return acts + (size_t)(begin + i) * ff; }, rows, W_down + ((size_t)e * hidden + c0) * ff, cols, ff,
+                  acc, lds);
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  if (tx >= cols) return;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = ty + 4 * i;
+    if (row < rows) {
+      const int pair = sorted[begin + row];
+      parts[((size_t)(pair % top) * num_tokens + pair / top) * hidden + c0 + tx] = wts[pair] * acc[i];
+    }
+  }
+}
+
+extern "C" int me_routed_ff_max_tiles(long long tokens, int E, int top) {
+  return (int)((tokens * top + TP_ROWS - 1) / TP_ROWS) + E;
+}
+
+// Bytes of workspace: ids and weights of the pairs, the tile list, the sorted pairs, the activations.
+extern "C" long long me_routed_ff_workspace(long long tokens, int E, int top, int ff, int elem) {
+  const long long P = tokens * top;
+  const long long ints = P + P + 1 + 3ll * me_routed_ff_max_tiles(tokens, E, top) + P;
+  return ints * 4 + 256 + P * ff * elem + 256;
+}
+
+// h [T, hidden] -> parts float32 [top, T, hidden]. Wr float32 [E, hidden]; W_gu [E, 2 ff, hidden]; W_down [E, hidden, ff].
+extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, const void* W_down, float* parts, void* workspace,
+                            int num_tokens, int hidden, int E, int top, int ff, int act, int dtype, hipStream_t stream) {
+  if (num_tokens <= 0) return 0;
+  if (E < 1 || E > RF_MAX_EXPERTS || top < 1 || top > RF_MAX_TOP || top > E)
+    return me_fail("me_routed_ff: %d experts (at most %d), %d of them a token (at most %d)", E, RF_MAX_EXPERTS, top, RF_MAX_TOP);
+  if (hidden <= 0 || ff <= 0) return me_fail("me_routed_ff: hidden=%d ff=%d", hidden, ff);
+  const long long P = (long long)num_tokens * top;
+  const int max_tiles = me_routed_ff_max_tiles(num_tokens, E, top);
+  int* ids = (int*)workspace;
+  float* wts = (float*)(ids + P);
+  int* plan = (int*)(wts + P);
+  int* sorted = plan + 1 + 3 * (size_t)max_tiles;
+  const size_t elem = dtype == ME_F32 ? 4 : 2;
+  char* acts = (char*)(((uintptr_t)(sorted + P) + 255) & ~(uintptr_t)255);
+  const dim3 g_up(max_tiles, (ff + TP_COLS - 1) / TP_COLS), g_down(max_tiles, (hidden + TP_COLS - 1) / TP_COLS);
+  if (g_up.y > 65535 || g_down.y > 65535) return me_fail("me_routed_ff: hidden=%d ff=%d", hidden, ff);
+  (void)elem;
+  if (dtype == ME_F32) {
+    routed_route_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)h, Wr, ids, wts, hidden, E, top);
+    routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, plan, sorted);
+    routed_gate_up_kernel<float><<<g_up, 256, 0, stream>>>((const float*)h, (const float*)W_gu, plan, sorted, (float*)acts, hidden, ff,
+                                                            top, act);
+    routed_down_kernel<float><<<g_down, 256, 0, stream>>>((const float*)acts, (const float*)W_down, plan, sorted, wts, parts,
+                                                          num_tokens, hidden, ff, top);
+  } else {
+    routed_route_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
+    routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, plan, sorted);
+    routed_gate_up_kernel<bf16_t><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, (bf16_t*)acts, hidden,
+                                                             ff, top, act);
+    routed_down_kernel<bf16_t><<<g_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, parts,
+                                                           num_tokens, hidden, ff, top);
+  }
+  return me_check_launch("me_routed_ff");
+}

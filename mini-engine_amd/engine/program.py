@@ -28,8 +28,10 @@ from ..ops.library import lib
 _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 _declared = False
 
-EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS, DECAY_STATE, HOLD = range(14)
-OP_INTS, OP_FLOATS = 16, 4  # csrc/host/program.h: kOpInts, kOpFloats
+(EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS, DECAY_STATE, HOLD, STREAMS,
+ STREAM_NORM, STREAM_HEAD, LATENT_ATTENTION, ROUTED_FF) = range(19)
+OP_PTRS, OP_INTS, OP_FLOATS = 8, 16, 4  # csrc/host/program.h: kOpPtrs, kOpInts, kOpFloats
+MAX_STREAMS = 8  # csrc/streams.hip: ME_MAX_STREAMS
 _RAISES = {1: ValueError, 2: RuntimeError, 3: AssertionError}
 
 
@@ -153,6 +155,8 @@ class StepProgram:
         self._held_value: int | None = None  # the value of a delta that was set aside (hold)
         self.num_ops = 0
         self.delta_scale = 1.0  # what the block being written multiplies its parts' results by (set by the block)
+        self.num_streams = 0  # residual streams of a token (0: the one plain stream)
+        self._stream_rewrite: torch.Tensor | None = None  # how the pending result rewrites the streams (mix, then out)
         self.draws = False
         self.last_prefill_columns = 0  # query columns of the prefill attention's blocks in the last eager step (0: none ran)
         # called parts: their C trampolines (kept alive), the memory and the batch of the step that is running,
@@ -205,7 +209,7 @@ class StepProgram:
 
     # -------------------------------------------------------------- operations
     def op(self, kind: int, in_: int = -1, out: int = -1, ptrs=(), ints=(), floats=()) -> None:
-        p = (ctypes.c_void_p * 6)()
+        p = (ctypes.c_void_p * OP_PTRS)()
         for i, t in enumerate(ptrs):
             if t is not None:
                 if not t.is_contiguous():
@@ -271,7 +275,8 @@ class StepProgram:
     def attention(self, qkv: int, *, q_norm: torch.Tensor | None, k_norm: torch.Tensor | None, rope: torch.Tensor | None,
                   k_cache: torch.Tensor, v_cache: torch.Tensor, heads: int, kv_heads: int, head_dim: int, block_size: int,
                   window: int, writes: bool, group: int, eps: float, scale: float, value_dim: int | None = None,
-                  keep_first: int = 0, pairing: int = 0, value_rope: torch.Tensor | None = None, value_pairing: int = 0) -> int:
+                  keep_first: int = 0, pairing: int = 0, value_rope: torch.Tensor | None = None, value_pairing: int = 0,
+                  query_temperature: tuple[float, int] | None = None, gated: bool = False) -> int:
         """Per-head q/k norm, rotation, page write and causal attention over the request's pages for a
         value ``[tokens, (heads + 2 kv_heads) head_dim]`` (``writes`` false: ``[tokens, heads head_dim]``,
         the pages are another layer's); returns the value ``[tokens, heads head_dim]``.
@@ -280,9 +285,14 @@ class StepProgram:
         heads of that size and the result has ``heads * value_dim`` columns); ``keep_first``: the first keys that stay
         visible behind the window; ``pairing``: 0 pairs element j with j + r/2, 1 pairs 2j with 2j + 1;
         ``value_rope`` / ``value_pairing``: the table ``[positions, 2, value_dim / 2]`` that the values are turned by
-        before they are cached and the outputs turned back by."""
+        before they are cached and the outputs turned back by; ``query_temperature`` ``(coef, every)``: the query at position p
+        is multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``; ``gated``: the input ends in one more column per head,
+        whose sigmoid multiplies the head's output."""
         dv = head_dim if value_dim is None else int(value_dim)
-        cols = heads * head_dim + (kv_heads * (head_dim + dv) if writes else 0)
+        cols = heads * head_dim + (kv_heads * (head_dim + dv) if writes else 0) + (heads if gated else 0)
+        coef, every = (0.0, 0) if query_temperature is None else (float(query_temperature[0]), int(query_temperature[1]))
+        if query_temperature is not None and every < 1:
+            raise ValueError("a temperature on the queries grows every so many positions, at least every one")
         if self._value_kinds[qkv] != (cols, self.elem):
             raise ValueError(f"the attention's input has {self._value_kinds[qkv][0]} columns, not {cols}")
         rotary_dim = covers = 0
@@ -300,9 +310,84 @@ class StepProgram:
         out = self.take(heads * dv)
         self.op(ATTENTION, in_=qkv, out=out, ptrs=[q_norm, k_norm, rope, k_cache, v_cache, value_rope],
                 ints=[heads, kv_heads, head_dim, rotary_dim, block_size, window, int(writes), group, covers,
-                      0 if dv == head_dim else dv, keep_first, pairing, turned],
-                floats=[eps, scale])
+                      0 if dv == head_dim else dv, keep_first, pairing, turned, every, int(gated)],
+                floats=[eps, scale, coef])
         return out
+
+    def latent_attention(self, proj: int, *, latent_norm: torch.Tensor, rope: torch.Tensor, k_cache: torch.Tensor,
+                         v_cache: torch.Tensor, key_map: torch.Tensor, value_map: torch.Tensor, sink: torch.Tensor | None,
+                         heads: int, head_dim: int, rotary_dim: int, rank: int, value_dim: int, block_size: int, group: int,
+                         eps: float, scale: float) -> int:
+        """Attention over one cached latent per token for a value ``[tokens, heads (head_dim + rotary_dim) | rank + rotary_dim |
+        heads]`` (queries; the latent projection and the key part that all heads share; a gate per head). ``key_map`` ``[heads,
+        rank, head_dim]`` (the keys' map per head, transposed) and ``value_map`` ``[heads, value_dim, rank]`` in the compute
+        dtype; ``sink`` float32 ``[heads]`` or None; pages of one key/value head with keys of ``rank + rotary_dim`` and values
+        of ``rank`` elements. Returns the value ``[tokens, heads * value_dim]``, gated."""
+        cols = heads * (head_dim + rotary_dim) + rank + rotary_dim + heads
+        if self._value_kinds[proj] != (cols, self.elem):
+            raise ValueError(f"the projections have {self._value_kinds[proj][0]} columns, not {cols}")
+        self._want(latent_norm, torch.float32, (rank,), "weight of the latent's norm")
+        self._want(rope, torch.float32, None, "rotary table")
+        if 2 * rope.shape[2] != rotary_dim or rope.shape[0] < self.max_positions:
+            raise ValueError(f"the rotary table must cover {self.max_positions} positions and {rotary_dim} elements")
+        self._want(key_map, self.dtype, (heads, rank, head_dim), "the keys' map")
+        self._want(value_map, self.dtype, (heads, value_dim, rank), "the values' map")
+        if sink is not None:
+            self._want(sink, torch.float32, (heads,), "sink")
+        if tuple(k_cache.shape[1:]) != (1, block_size, rank + rotary_dim) or tuple(v_cache.shape[1:]) != (1, rank, block_size):
+            raise ValueError("a latent attention layer keeps pages of one head: keys of rank + rotary_dim, values of rank elements")
+        out = self.take(heads * value_dim)
+        self.op(LATENT_ATTENTION, in_=proj, out=out, ptrs=[latent_norm, rope, k_cache, v_cache, key_map, value_map, sink],
+                ints=[heads, head_dim, rotary_dim, rank, value_dim, block_size, group, rope.shape[0]], floats=[eps, scale])
+        return out
+
+    def routed_ff(self, x: int, *, router: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, top_k: int, activation: str) -> None:
+        """A feed-forward of routed experts on the value ``x`` as the part's result. ``router`` float32 ``[experts, hidden]``;
+        ``gate_up`` ``[experts, 2 ff, hidden]`` (an expert's gate rows, then its up rows) and ``down`` ``[experts, hidden, ff]``
+        in the compute dtype."""
+        from ..ops.kernels import gate_code
+
+        experts, two_ff, hidden = gate_up.shape
+        if self._value_kinds[x] != (self.hidden, self.elem) or hidden != self.hidden:
+            raise ValueError("routed experts read the hidden size in the compute dtype")
+        self._want(router, torch.float32, (experts, hidden), "router")
+        self._want(gate_up, self.dtype, None, "experts' gate and up rows")
+        self._want(down, self.dtype, (experts, hidden, two_ff // 2), "experts' down rows")
+        if not 1 <= top_k <= experts:
+            raise ValueError(f"{top_k} of {experts} experts a token")
+        self.op(ROUTED_FF, in_=x, ptrs=[router, gate_up, down], ints=[experts, top_k, two_ff // 2, gate_code(activation)])
+        self._pending_value = None
+
+    # ----------------------------------------------------------- several residual streams
+    def spread_streams(self, streams: int) -> None:
+        """From here on every token has ``streams`` residual streams, each a copy of the stream as it is now."""
+        if not 1 <= streams <= MAX_STREAMS:
+            raise ValueError(f"1 to {MAX_STREAMS} residual streams are taken, not {streams}")
+        if self.num_streams:
+            raise ValueError("the streams are spread once")
+        self.op(STREAMS, ints=[streams])
+        self.num_streams = int(streams)
+
+    def stream_normed(self, norm, reads: torch.Tensor) -> int:
+        """The input of the coming part as a value: the pending result rewrites the streams (by what :meth:`rewrites_streams`
+        said of it), ``sum_s reads[s] x_s`` is normed by ``norm`` (RMS-shaped)."""
+        weight, eps = norm.as_fused()
+        if getattr(norm, "groups", 1) != 1:
+            raise ValueError("the norm over several streams is not cut into groups")
+        self._want(weight, torch.float32, (self.hidden,), "norm weight")
+        self._want(reads, torch.float32, (self.num_streams,), "what a part reads of the streams")
+        out = self.take(self.hidden, self.elem)
+        self.op(STREAM_NORM, out=out, ptrs=[weight, self._stream_rewrite, reads], floats=[eps])
+        self._stream_rewrite = None
+        self.pending_consumed()
+        return out
+
+    def rewrites_streams(self, mix_out: torch.Tensor) -> None:
+        """The result that is pending now rewrites the streams by ``mix_out`` float32 ``[S * S + S]``: ``mix[from, to]``, then
+        ``out[to]``."""
+        s = self.num_streams
+        self._want(mix_out, torch.float32, (s * s + s,), "how a result rewrites the streams")
+        self._stream_rewrite = mix_out
 
     def decay_state(self, proj: int, *, decay: torch.Tensor, rope: torch.Tensor | None, pairing: int, norm_weight: torch.Tensor | None,
                     state: torch.Tensor, heads: int, key_dim: int, value_dim: int, input_act: int, key_scale: float,
@@ -359,7 +444,7 @@ class StepProgram:
 
         c_fn = _CALL_FN(trampoline)
         self._calls.append(c_fn)
-        p = (ctypes.c_void_p * 6)()
+        p = (ctypes.c_void_p * OP_PTRS)()
         p[0] = ctypes.cast(c_fn, ctypes.c_void_p).value
         iv, fv = (ctypes.c_int64 * OP_INTS)(), (ctypes.c_float * OP_FLOATS)()
         self.num_ops = _ok(self._L.me_runner_op(self.handle, CALL, in_, out, p, iv, fv))
@@ -395,7 +480,13 @@ class StepProgram:
         """Final norm of the wanted rows, the head product, the logits times ``logit_scale``."""
         norm_weight, eps = norm.as_fused()
         self._want(weight, self.dtype, (self.vocab, self.hidden), "head")
-        self.op(HEAD, ptrs=[norm_weight, weight], ints=[getattr(norm, "groups", 1)], floats=[eps, logit_scale])
+        if self.num_streams:  # the streams' sum, with the pending rewrite applied to the wanted rows
+            if getattr(norm, "groups", 1) != 1:
+                raise ValueError("the norm over several streams is not cut into groups")
+            self.op(STREAM_HEAD, ptrs=[norm_weight, weight, self._stream_rewrite], floats=[eps, logit_scale])
+            self._stream_rewrite = None
+        else:
+            self.op(HEAD, ptrs=[norm_weight, weight], ints=[getattr(norm, "groups", 1)], floats=[eps, logit_scale])
         self.pending_consumed()
 
     def sample(self) -> None:

@@ -1,6 +1,6 @@
 """Parts of a decoder layer. Importing this package registers the built-in kinds."""
 
-from . import attention, decay_state, mlp, norm, rotary  # noqa: F401
+from . import attention, decay_state, latent_attention, mlp, norm, rotary, routed_experts  # noqa: F401
 from .base import (
     BLOCK_ARRANGEMENTS,
     FEED_FORWARDS,
@@ -16,7 +16,7 @@ from .base import (
     StateBinding,
     StateNeed,
 )
-from .block import ParallelBlock, PreNormBlock, build_block
+from .block import HyperConnectionBlock, ParallelBlock, PreNormBlock, build_block
 from .decoder import Decoder
 
 __all__ = [
@@ -24,6 +24,7 @@ __all__ = [
     "Decoder",
     "FEED_FORWARDS",
     "FeedForward",
+    "HyperConnectionBlock",
     "KVBinding",
     "KVCacheNeed",
     "MIXERS",

@@ -52,8 +52,14 @@ class Attention(Mixer):
         if self.value_position is not None and self.value_position.rotary_dim != self.dv:
             raise ValueError(f"values of size {self.dv} are turned over all of their elements, not {self.value_position.rotary_dim}")
         self.pairing = 0 if self.position is None else int(getattr(self.position, "pairing_code", 0))
+        self.q_temp = getattr(s, "query_temperature", None)
+        if self.q_temp is not None and int(self.q_temp[1]) < 1:
+            raise ValueError(f"a temperature on the queries grows every {self.q_temp[1]} positions: at least every one")
+        self.gated = bool(getattr(s, "output_gate", False))
+        self.norm_weighted = bool(getattr(s, "qk_norm_weight", True))
         # the plain form: what the matrix-core kernels and the fused decode prologue are written for
-        self.plain = self.dv == self.d and not self.keep_first and self.pairing == 0 and self.value_position is None
+        self.plain = (self.dv == self.d and not self.keep_first and self.pairing == 0 and self.value_position is None
+                      and self.q_temp is None and not self.gated)
         if self.plain and (s.head_dim % 16 or not 16 <= s.head_dim <= MAX_HEAD_DIM):
             raise ValueError(f"head_dim={s.head_dim} is not supported: the attention kernels take head sizes "
                              f"from 16 to {MAX_HEAD_DIM} in steps of 16")
@@ -65,7 +71,7 @@ class Attention(Mixer):
         names = dict(getattr(s, "names", ()) or ())
         self._n = {r: names.get(r, d) for r, d in (("q", "q_proj.weight"), ("k", "k_proj.weight"), ("v", "v_proj.weight"),
                                                     ("o", "o_proj.weight"), ("q_norm", "q_norm.weight"),
-                                                    ("k_norm", "k_norm.weight"))}
+                                                    ("k_norm", "k_norm.weight"), ("g", "g_proj.weight"))}
         self.q_norm_w = self.k_norm_w = None
         self.w_qkv = self.w_o = None
 
@@ -80,24 +86,28 @@ class Attention(Mixer):
         if s.cache_from is None:
             wants[f"{prefix}.{n['k']}"] = TensorWant((s.num_kv_heads * s.head_dim, s.hidden_size))
             wants[f"{prefix}.{n['v']}"] = TensorWant((s.num_kv_heads * self.dv, s.hidden_size))
-        if s.qk_norm_eps is not None:
+        if s.qk_norm_eps is not None and self.norm_weighted:
             wants[f"{prefix}.{n['q_norm']}"] = TensorWant((s.head_dim,), "vector")
             if s.cache_from is None:
                 wants[f"{prefix}.{n['k_norm']}"] = TensorWant((s.head_dim,), "vector")
+        if self.gated:
+            wants[f"{prefix}.{n['g']}"] = TensorWant((s.num_heads, s.hidden_size))
         return wants
 
     def load(self, tensors, prefix: str) -> None:
         s = self.spec
         n = self._n
         q = tensors[f"{prefix}.{n['q']}"]
-        if s.cache_from is None:
-            self.w_qkv = torch.cat((q, tensors[f"{prefix}.{n['k']}"], tensors[f"{prefix}.{n['v']}"]), dim=0)
-        else:
-            self.w_qkv = q.contiguous()
+        rows = [q] if s.cache_from is not None else [q, tensors[f"{prefix}.{n['k']}"], tensors[f"{prefix}.{n['v']}"]]
+        if self.gated:  # the gates' rows ride behind q, k and v: one product for all
+            rows.append(tensors[f"{prefix}.{n['g']}"])
+        self.w_qkv = torch.cat(rows, dim=0) if len(rows) > 1 else q.contiguous()
         self.w_o = tensors[f"{prefix}.{n['o']}"]
-        if s.qk_norm_eps is not None:
+        if s.qk_norm_eps is not None and self.norm_weighted:
             self.q_norm_w = tensors[f"{prefix}.{n['q_norm']}"]
             self.k_norm_w = tensors.get(f"{prefix}.{n['k_norm']}")
+        elif s.qk_norm_eps is not None:  # the norm has no weight: the kernels multiply by ones
+            self.q_norm_w = self.k_norm_w = torch.ones(s.head_dim, dtype=torch.float32, device=q.device)
 
     # ---- cache
     def cache_need(self):
@@ -118,6 +128,8 @@ class Attention(Mixer):
         if b is None:
             raise RuntimeError("attention mixer was given no cache")
         owns = s.cache_from is None
+        if self.q_temp is not None or self.gated:
+            raise NotImplementedError("a temperature on the queries and an output gate run in the step program only")
         proj = K.linear(h, self.w_qkv)  # [T, (nh + 2 nkv) d] or [T, nh d]
         table = batch.block_table(b.group)
         rope = None if self.position is None else self.position.tables(batch.max_ctx)
@@ -181,7 +193,8 @@ class Attention(Mixer):
             eps=0.0 if s.qk_norm_eps is None else float(s.qk_norm_eps), scale=float(s.scale),
             value_dim=self.dv, keep_first=self.keep_first, pairing=self.pairing,
             value_rope=None if self.value_position is None else self.value_position.tables(program.max_positions),
-            value_pairing=0 if self.value_position is None else self.value_position.pairing_code)
+            value_pairing=0 if self.value_position is None else self.value_position.pairing_code,
+            query_temperature=self.q_temp, gated=self.gated)
         program.linear_delta(out, self.w_o)
 
     def attend(self, q: torch.Tensor, batch, table: torch.Tensor, b: KVBinding) -> torch.Tensor:

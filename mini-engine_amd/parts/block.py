@@ -113,8 +113,83 @@ class ParallelBlock:
                 program.delta_scale = before
 
 
+class HyperConnectionBlock:
+    """The pre-norm arrangement over several residual streams (hyper-connections). A part (the mixer, then the feed-forward,
+    which may be absent) reads ``u = sum_s in[s] x_s``, gives ``y = part(norm(u))``, and all streams are rewritten at once
+    from the old ones: ``x_t = sum_s mix[s, t] x_s + out[t] y``. The coefficients are tensors of the checkpoint (the layer
+    spec's ``mixer_streams`` / ``ffn_streams`` name them), kept in float32. The rewrite rides on the kernel that reads and
+    norms the next part's input, as the single stream's add rides on its next norm."""
+
+    def __init__(self, spec, dtype: torch.dtype, device: torch.device):
+        self.spec, self.dtype = spec, dtype
+        self.mixer = MIXERS.build(spec.mixer, dtype, device)
+        self.ffn = None if spec.ffn is None else FEED_FORWARDS.build(spec.ffn, dtype, device)
+        self.mixer_norm = NORMS.build(spec.mixer_norm, dtype, device)
+        self.ffn_norm = None if spec.ffn is None else NORMS.build(spec.ffn_norm, dtype, device)
+        if spec.mixer_streams is None or (self.ffn is not None and spec.ffn_streams is None):
+            raise ValueError("every part of a hyper-connection block needs its stream coefficients")
+        for norm in (self.mixer_norm, self.ffn_norm):
+            if norm is not None and (norm.as_fused() is None or getattr(norm, "groups", 1) != 1):
+                raise ValueError("the parts of a hyper-connection block are normed by an RMS norm without groups")
+        self.reads: dict[str, torch.Tensor] = {}
+        self.rewrites: dict[str, torch.Tensor] = {}
+
+    def _ties(self):
+        s = self.spec
+        return [s.mixer_streams] + ([s.ffn_streams] if self.ffn is not None else [])
+
+    def weight_wants(self):
+        from ..weights.loader import TensorWant
+
+        s = self.spec
+        wants = {}
+        wants.update(self.mixer_norm.weight_wants(s.mixer_norm_name))
+        wants.update(self.mixer.weight_wants(s.mixer_prefix))
+        if self.ffn is not None:
+            wants.update(self.ffn_norm.weight_wants(s.ffn_norm_name))
+            wants.update(self.ffn.weight_wants(s.ffn_prefix))
+        for tie in self._ties():
+            n = int(tie.streams)
+            wants[f"{tie.prefix}.in"] = TensorWant((n,), "vector")
+            wants[f"{tie.prefix}.out"] = TensorWant((n,), "vector")
+            wants[f"{tie.prefix}.mix"] = TensorWant((n, n), "vector")
+        return wants
+
+    def load(self, tensors) -> None:
+        s = self.spec
+        self.mixer_norm.load(tensors, s.mixer_norm_name)
+        self.mixer.load(tensors, s.mixer_prefix)
+        if self.ffn is not None:
+            self.ffn_norm.load(tensors, s.ffn_norm_name)
+            self.ffn.load(tensors, s.ffn_prefix)
+        for tie in self._ties():
+            self.reads[tie.prefix] = tensors[f"{tie.prefix}.in"].contiguous()
+            # mix[from, to] row by row, then out[to]: what the kernel that rewrites the streams reads
+            self.rewrites[tie.prefix] = torch.cat((tensors[f"{tie.prefix}.mix"].reshape(-1), tensors[f"{tie.prefix}.out"])).contiguous()
+
+    def emit(self, program, cache=None) -> None:
+        s = self.spec
+        parts = [(self.mixer, self.mixer_norm, s.mixer_streams, (cache,))]
+        if self.ffn is not None:
+            parts.append((self.ffn, self.ffn_norm, s.ffn_streams, ()))
+        for part, norm, tie, extra in parts:
+            if int(tie.streams) != program.num_streams:
+                raise ValueError(f"a block of {tie.streams} streams in a model of {program.num_streams}")
+            with program.scope():
+                h = program.stream_normed(norm, self.reads[tie.prefix])
+                if callable(getattr(part, "emit", None)):
+                    out = part.emit(program, h, *extra)
+                else:
+                    out = program.call(lambda frame, part=part, extra=extra: frame.write(part.forward(frame.input, frame.batch, *extra)),
+                                       in_=h, out_cols=program.hidden)
+                if out is not None:
+                    program.delta(out)
+                program.rewrites_streams(self.rewrites[tie.prefix])
+
+
 BLOCK_ARRANGEMENTS.register("pre_norm", PreNormBlock)
 BLOCK_ARRANGEMENTS.register("parallel", ParallelBlock)
+BLOCK_ARRANGEMENTS.register("hyper_connections", HyperConnectionBlock)
 
 
 def build_block(spec, dtype, device):

@@ -88,6 +88,8 @@ class Decoder:
         if self.embed_table is None:
             raise RuntimeError("weights are not loaded")
         program.embed(self.embed_table, self.plan.embedding_multiplier or 1.0)
+        if getattr(self.plan, "residual_streams", 0):
+            program.spread_streams(int(self.plan.residual_streams))
         for r, i in enumerate(self.plan.order):
             self.blocks[i].emit(program, self.bindings[r])
         if self.final_norm.as_fused() is not None:

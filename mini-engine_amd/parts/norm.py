@@ -1,6 +1,8 @@
 """RMSNorm part: ``x * rsqrt(mean(x^2) + eps) * weight`` in float32
 (reference: ``src/mini_engine/model.py:59-69``; the weight multiplies directly, eps inside the root). With
-``groups > 1`` the row is cut into that many equal consecutive parts and each is divided by its own root mean square."""
+``groups > 1`` the row is cut into that many equal consecutive parts and each is divided by its own root mean square.
+With ``weight_offset`` the stored weight lies that far below the one that multiplies (weights stored around zero): the
+offset is added once, in float32, when the weight is loaded."""
 
 from __future__ import annotations
 
@@ -19,6 +21,7 @@ class RMSNorm(Norm):
         self.eps = float(spec.eps)
         self.dim = int(spec.dim)
         self.groups = int(getattr(spec, "groups", 1))
+        self.weight_offset = float(getattr(spec, "weight_offset", 0.0))
         if self.groups < 1 or self.dim % self.groups:
             raise ValueError(f"a norm over {self.dim} elements cannot be cut into {self.groups} equal groups")
         self.weight = torch.ones(self.dim, dtype=torch.float32, device=device)
@@ -27,7 +30,7 @@ class RMSNorm(Norm):
         return {name: TensorWant((self.dim,), "vector")}
 
     def load(self, tensors, name: str) -> None:
-        self.weight = tensors[name]
+        self.weight = tensors[name] + self.weight_offset if self.weight_offset else tensors[name]
 
     def as_fused(self):
         return self.weight, self.eps

@@ -56,6 +56,52 @@ class Rotary(PositionEncoding):
         return self._table
 
 
+class YarnRotary(PositionEncoding):
+    """Rotation of pairs of halves whose slow pairs are stretched by a factor, the fast ones left alone and those between
+    blended (the spec says how); cosines and sines carry the encoding's multiplier. The table is worked out in double
+    precision on the host and rounded once."""
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        import math
+
+        rd, base = int(spec.rotary_dim), float(spec.theta)
+        if rd <= 0 or rd % 2:
+            raise ValueError(f"rotary_dim must be a positive even number, got {rd}")
+        if getattr(spec, "pairing", "halves") != "halves":
+            raise ValueError("the stretched rotation pairs halves")
+        factor, original = float(spec.factor), float(spec.original)
+        if not (factor > 0.0 and original > 0.0 and float(spec.fast) > 0.0 and float(spec.slow) > 0.0 and base > 1.0):
+            raise ValueError("factor, original, fast and slow must be positive and the base above 1")
+        self.rotary_dim, self.pairing, self.pairing_code = rd, "halves", 0
+        j = torch.arange(rd // 2, dtype=torch.float64)
+        freq = torch.exp(-(2.0 * j / rd) * math.log(base))
+
+        def pair_of(turns: float) -> float:
+            return rd * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+        lo = max(math.floor(pair_of(float(spec.fast))), 0)
+        hi = min(math.ceil(pair_of(float(spec.slow))), rd - 1)
+        ramp = ((j - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        self.freq = freq / factor * ramp + freq * (1.0 - ramp)
+        self.multiplier = 0.1 * math.log(factor) + 1.0
+        self._table: torch.Tensor | None = None
+        self._retired: list[torch.Tensor] = []
+
+    def tables(self, num_positions: int = 1) -> torch.Tensor:
+        if self._table is None or self._table.shape[0] < num_positions:
+            size = 256
+            while size < num_positions:
+                size *= 2
+            if self._table is not None:
+                self._retired.append(self._table)  # a captured graph may still read the smaller table
+            ang = torch.arange(size, dtype=torch.float64)[:, None] * self.freq[None, :]
+            table = torch.stack((torch.cos(ang), torch.sin(ang)), dim=1) * self.multiplier
+            self._table = table.to(torch.float32).contiguous().to(self.device)
+        return self._table
+
+
 PAIRINGS = {"halves": 0, "neighbours": 1}
 
 POSITION_ENCODINGS.register("rotary", Rotary)
+POSITION_ENCODINGS.register("yarn_rotary", YarnRotary)
