@@ -1182,3 +1182,141 @@ def unturn_rows(rows: torch.Tensor, table: torch.Tensor, pairing: int, positions
                                _stream()))
     return rows
 
+
+
+# ------------------------------------------------------------------ several residual streams
+_i64 = ctypes.c_longlong
+
+
+def streams_norm(xs: torch.Tensor, delta, rewrite: torch.Tensor | None, reads: torch.Tensor | None, weight: torch.Tensor,
+                 eps: float, out_dtype: torch.dtype, rows: torch.Tensor | None = None, write_x: bool = True) -> torch.Tensor:
+    """``xs`` float32 ``[S, T, dim]`` (rewritten in place when ``write_x``): the pending result ``delta`` (a tensor ``[T, dim]`` in
+    ``out_dtype``, or :class:`PartialSums`) rewrites the streams by ``rewrite`` float32 ``[S * S + S]`` (``mix[from, to]`` row by
+    row, then ``out[to]``); then ``sum_s reads[s] xs[s]`` (``reads`` None: ones) of every row (or of ``rows``) is RMS-normed with
+    ``weight``. Returns the normed rows in ``out_dtype``."""
+    _want(xs, "xs", torch.float32, (None, None, None))
+    s, t, dim = xs.shape
+    _want(weight, "weight", torch.float32, (dim,))
+    parts = delta if isinstance(delta, PartialSums) else None
+    tensor = None if parts is not None else delta
+    if tensor is not None:
+        _want(tensor, "delta", out_dtype, (t, dim))
+    if parts is not None:
+        _want(parts.parts, "partial sums", torch.float32, (None, t, dim))
+    if rewrite is not None:
+        _want(rewrite, "rewrite", torch.float32, (s * s + s,))
+    if reads is not None:
+        _want(reads, "reads", torch.float32, (s,))
+    n = t if rows is None else int(rows.shape[0])
+    if rows is not None:
+        _want(rows, "rows", torch.int32, (n,))
+    out = torch.empty((n, dim), dtype=out_dtype, device=xs.device)
+    check(lib().me_streams_norm(
+        _p(xs), _i64(t * dim), _i(s), _p(tensor), _p(None if parts is None else parts.parts), _i(0 if parts is None else parts.parts.shape[0]),
+        _i64(t * dim), _p(rewrite), _p(reads), _p(weight), _p(out), _p(rows), _i(n), _i(dim), _f(eps), _i(int(write_x)),
+        _i(_code(out_dtype)), _stream()))
+    return out
+
+
+def streams_spread(xs: torch.Tensor) -> torch.Tensor:
+    """``xs`` float32 ``[S, T, dim]``: every stream becomes a copy of the first."""
+    _want(xs, "xs", torch.float32, (None, None, None))
+    check(lib().me_streams_spread(_p(xs), _i64(xs.shape[1] * xs.shape[2]), _i(xs.shape[0]), _stream()))
+    return xs
+
+
+# ------------------------------------------------------------------ attention with a sink, a gate, a temperature
+def attention_gated(q, k_cache, v_cache, positions, token_item, block_table, scale: float, sink: torch.Tensor | None = None,
+                    gate: torch.Tensor | None = None, window: int = 0) -> torch.Tensor:
+    """As :func:`attention_general` (the kernel with a wave per token and head), with ``sink`` float32 ``[nh]`` in the
+    softmax's denominator and every head's output times the sigmoid of ``gate`` ``[T, nh]`` (the activations' dtype)."""
+    _want(q, "q", None, (None, None, None))
+    t, nh, d = q.shape
+    nkv, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
+    _check_cache(k_cache, v_cache, q.dtype, nkv, d, bs, dv)
+    _check_step_index(positions, token_item, block_table, t)
+    if sink is not None:
+        _want(sink, "sink", torch.float32, (nh,))
+    if gate is not None:
+        _want(gate, "gate", q.dtype, (t, nh))
+    out = torch.empty((t, nh * dv), dtype=q.dtype, device=q.device)
+    check(lib().me_attention_general_gated(
+        _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]), _p(out), _i(t),
+        _i(nh), _i(nkv), _i(d), _i(dv), _i(bs), _i(window), _i(0), _p(None), _i(0), _f(scale), _p(sink), _p(gate), _i64(nh),
+        _i(_code(q.dtype)), _i(0), _stream()))
+    return out
+
+
+def qkv_scatter_rows(qkv, q_w, k_w, positions, token_item, block_table, k_cache, v_cache, nh: int, nkv: int, d: int, dv: int,
+                     eps: float, q_temp: tuple[float, int] | None = None, extra_columns: int = 0) -> torch.Tensor:
+    """q/k norm and page write without rotation for rows ``[T, nh d + nkv d + nkv dv + extra_columns]`` (the extra columns are
+    not read), every query times ``1 + coef * ln(floor((position + 1) / every) + 1)`` for ``q_temp = (coef, every)``; returns q
+    ``[T, nh, d]``."""
+    t = qkv.shape[0]
+    width = (nh + nkv) * d + nkv * dv + extra_columns
+    _want(qkv, "qkv", None, (t, width))
+    _check_cache(k_cache, v_cache, qkv.dtype, nkv, d, k_cache.shape[2], dv)
+    _check_step_index(positions, token_item, block_table, t)
+    q = torch.empty((t, nh, d), dtype=qkv.dtype, device=qkv.device)
+    coef, every = (0.0, 0) if q_temp is None else q_temp
+    check(lib().me_qkv_rotate_scatter_rows(
+        _p(qkv), _i64(width if extra_columns else 0), _p(q_w), _p(k_w), _p(None), _i(0), _i(0), _p(None), _i(0), _f(coef), _i(every),
+        _p(positions), _p(token_item), _p(block_table), _i(block_table.shape[1]), _p(q), _p(k_cache), _p(v_cache), _i(t), _i(nh),
+        _i(nkv), _i(d), _i(dv), _i(k_cache.shape[2]), _f(eps), _i(_code(qkv.dtype)), _p(None), _i(0), _i(0), _stream()))
+    return q
+
+
+# ------------------------------------------------------------------ attention over cached latents
+def latent_prepare(proj, norm_w, rope, positions, token_item, block_table, k_cache, v_cache, nh: int, d: int, r: int, rank: int,
+                   eps: float) -> torch.Tensor:
+    """The latent's norm, the rotation and the page write for rows ``[T, nh (d + r) | rank + r | ...]``; returns qa ``[T, nh,
+    rank + r]`` whose last ``r`` elements per head are the turned query parts (the first ``rank`` are left for
+    :func:`head_product`)."""
+    t = proj.shape[0]
+    _want(proj, "proj", None, (t, None))
+    _want(norm_w, "norm weight", torch.float32, (rank,))
+    _want(rope, "rope", torch.float32, (None, 2, r // 2))
+    _check_step_index(positions, token_item, block_table, t)
+    bs = k_cache.shape[2]
+    _check_cache(k_cache, v_cache, proj.dtype, 1, rank + r, bs, rank)
+    qa = torch.zeros((t, nh, rank + r), dtype=proj.dtype, device=proj.device)
+    check(lib().me_latent_prepare(_p(proj), _i64(proj.shape[1]), _p(norm_w), _p(rope), _p(positions), _p(token_item), _p(block_table),
+                                  _i(block_table.shape[1]), _p(qa), _p(k_cache), _p(v_cache), _i(t), _i(nh), _i(d), _i(r), _i(rank),
+                                  _i(rank), _i(bs), _f(eps), _i(_code(proj.dtype)), _stream()))
+    return qa
+
+
+def head_product(x: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor | None = None) -> torch.Tensor:
+    """``out[t, h, :] = weight[h] @ x[t, h, :]`` for x ``[T, heads, k]`` (any strides of tokens and heads, elements contiguous) and
+    weight ``[heads, n, k]``, times the sigmoid of ``gate[t, h]`` if given. Returns ``[T, heads, n]``."""
+    t, heads, k = x.shape
+    _want(weight, "weight", x.dtype, (heads, None, k))
+    if x.stride(2) != 1:
+        raise ValueError("the elements of a head lie side by side")
+    n = weight.shape[1]
+    out = torch.empty((t, heads, n), dtype=x.dtype, device=x.device)
+    if gate is not None:
+        _want(gate, "gate", x.dtype, (t, heads))
+    check(lib().me_head_product(_p(x), _i64(x.stride(0)), _i64(x.stride(1)), _p(weight), _p(out), _i64(heads * n), _i64(n), _p(gate),
+                                _i64(heads), _i(t), _i(heads), _i(n), _i(k), _i(_code(x.dtype)), _stream()))
+    return out
+
+
+# ------------------------------------------------------------------ routed experts
+def routed_ff(h: torch.Tensor, router: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, top_k: int,
+              activation: str = "silu") -> PartialSums:
+    """The feed-forward of routed experts for h ``[T, hidden]``: float32 partial sums ``[top_k, T, hidden]``, one per pick of a
+    token in the order of the picks. ``router`` float32 ``[E, hidden]``, ``gate_up`` ``[E, 2 ff, hidden]``, ``down`` ``[E, hidden,
+    ff]``."""
+    t, hidden = h.shape
+    e, two_ff, _ = gate_up.shape
+    _want(router, "router", torch.float32, (e, hidden))
+    _want(gate_up, "gate_up", h.dtype, (e, two_ff, hidden))
+    _want(down, "down", h.dtype, (e, hidden, two_ff // 2))
+    lib().me_routed_ff_workspace.restype = ctypes.c_longlong
+    need = lib().me_routed_ff_workspace(_i64(t), _i(e), _i(top_k), _i(two_ff // 2), _i(h.element_size()))
+    ws = torch.empty(int(need), dtype=torch.uint8, device=h.device)
+    parts = torch.empty((top_k, t, hidden), dtype=torch.float32, device=h.device)
+    check(lib().me_routed_ff(_p(h), _p(router), _p(gate_up), _p(down), _p(parts), _p(ws), _i(t), _i(hidden), _i(e), _i(top_k),
+                             _i(two_ff // 2), _i(gate_code(activation)), _i(_code(h.dtype)), _stream()))
+    return PartialSums(parts)

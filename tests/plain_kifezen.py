@@ -133,11 +133,15 @@ def gated_ff(h: torch.Tensor, w: dict, pre: str) -> torch.Tensor:
     return (silu(h @ w[pre + ".gate"].T) * (h @ w[pre + ".up"].T)) @ w[pre + ".down"].T
 
 
-def routed_ff(h: torch.Tensor, mlp: dict, w: dict, pre: str) -> torch.Tensor:
-    """Every token: the ``top`` experts of the largest router logits, weighted by the softmax over those logits."""
+def routed_ff(h: torch.Tensor, mlp: dict, w: dict, pre: str, gaps: list | None = None) -> torch.Tensor:
+    """Every token: the ``top`` experts of the largest router logits, weighted by the softmax over those logits. ``gaps``
+    collects, per token, how far the last picked logit lies above the first one left out, as a share of the largest."""
     top = int(mlp["router"]["top"])
     z = h @ w[pre + ".router"].T
     val, idx = torch.topk(z, top, dim=-1)
+    if gaps is not None and top < z.shape[-1]:
+        ranked = z.sort(dim=-1, descending=True).values
+        gaps.append((ranked[:, top - 1] - ranked[:, top]) / z.abs().amax(dim=-1))
     wt = torch.softmax(val, dim=-1)
     out = torch.zeros(h.shape[0], w[pre + ".e0.down"].shape[0], dtype=F)
     for t in range(h.shape[0]):
@@ -149,21 +153,25 @@ def routed_ff(h: torch.Tensor, mlp: dict, w: dict, pre: str) -> torch.Tensor:
 MIXERS = {"attention": softmax_attention, "latent_attention": latent_attention}
 
 
-def forward(cfg: dict, w: dict, tokens: list[int], layer_outputs: list | None = None) -> torch.Tensor:
-    """Logits [T, vocab] of a whole sequence; ``layer_outputs`` collects the sum of the streams behind every layer."""
+def forward(cfg: dict, w: dict, tokens: list[int], layer_outputs: list | None = None, router_gaps: list | None = None,
+            after_norm=None) -> torch.Tensor:
+    """Logits [T, vocab] of a whole sequence; ``layer_outputs`` collects the sum of the streams behind every layer,
+    ``router_gaps`` every routed layer's gaps (:func:`routed_ff`); ``after_norm`` (a function) is applied to every part's
+    normed input (a rounding, to see how far a sequence's logits move under it)."""
+    after_norm = after_norm or (lambda z: z)
     eps, s = float(cfg["norm"]["eps"]), int(cfg.get("streams", 1))
     x = w["embed"][torch.tensor(tokens, dtype=torch.long)]
     streams = x[None].repeat(s, 1, 1)
     for i, layer in enumerate(cfg["layers"]):
         pre = f"l{i}"
         u = streams_read(streams, w[pre + ".hc1.in"])
-        y = MIXERS[layer["type"]](offset_norm(u, w[pre + ".norm1"], eps), layer["mixer"], w, pre + ".mix", eps)
+        y = MIXERS[layer["type"]](after_norm(offset_norm(u, w[pre + ".norm1"], eps)), layer["mixer"], w, pre + ".mix", eps)
         streams = streams_write(streams, y, w[pre + ".hc1.mix"], w[pre + ".hc1.out"])
         mlp = layer.get("mlp")
         if mlp is not None:
             u = streams_read(streams, w[pre + ".hc2.in"])
-            hn = offset_norm(u, w[pre + ".norm2"], eps)
-            y = gated_ff(hn, w, pre + ".mlp") if mlp["kind"] == "dense" else routed_ff(hn, mlp, w, pre + ".mlp")
+            hn = after_norm(offset_norm(u, w[pre + ".norm2"], eps))
+            y = gated_ff(hn, w, pre + ".mlp") if mlp["kind"] == "dense" else routed_ff(hn, mlp, w, pre + ".mlp", router_gaps)
             streams = streams_write(streams, y, w[pre + ".hc2.mix"], w[pre + ".hc2.out"])
         if layer_outputs is not None:
             layer_outputs.append(streams.sum(dim=0))
