@@ -141,9 +141,9 @@ class LatentAttentionSpec:
 
     @property
     def kv_elements_per_token(self) -> int:
-        """Elements one token occupies in this layer's pages: the key ``[c | shared part]`` and its value rows, the latent
-        once more."""
-        return 2 * self.latent_rank + self.rotary_dim
+        """Elements one token occupies in this layer's pages at most: the key ``[c | shared part]`` and its value rows (the
+        latent once more; the whole key once more where the matrix-core kernels serve the layer)."""
+        return 2 * (self.latent_rank + self.rotary_dim)
 
 
 @dataclass(frozen=True)

@@ -188,7 +188,7 @@ __device__ __forceinline__ void attention_decode_body(
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
     float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out, int nh, int nkv, int bs_shift,
     int window, float scale_log2, int num_splits, int head_chunks, const DecodeFusedArgs& fa,
-    const int* __restrict__ live_items, int waves_wanted) {
+    const int* __restrict__ live_items, int waves_wanted, const float* __restrict__ sink) {
   extern __shared__ float decode_lds[];  // only with several waves a block: their results, to be added up
   const int bs = 1 << bs_shift;
   const int item = blockIdx.x;
@@ -426,6 +426,12 @@ __device__ __forceinline__ void attention_decode_body(
     }
     const size_t head = (size_t)item * nh + head0 + hr;
     if (blocks_z == 1) {
+      if (sink) {  // one more term exp(sink) in the denominator, with no value (statistics are in units of log2)
+        const float s2 = sink[head0 + hr] * LOG2E, top = fmaxf(big, s2);
+        const float keep = big == -INFINITY ? 0.f : fast_exp2(big - top);
+        denom = denom * keep + fast_exp2(s2 - top);
+        total[0] *= keep, total[1] *= keep, total[2] *= keep, total[3] *= keep;
+      }
       const float inv = denom > 0.f ? 1.f / denom : 0.f;  // no visible key at all: zeros, not NaN
       *reinterpret_cast<short4_t*>(out + head * D + quad * 4) =
           pack_bf16x4(total[0] * inv, total[1] * inv, total[2] * inv, total[3] * inv);
@@ -450,17 +456,18 @@ __global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_k
     const int* __restrict__ item_ctx, const int* __restrict__ block_table, int table_width,
     float* __restrict__ part_o, float* __restrict__ part_ml, bf16_t* __restrict__ out, int nh, int nkv, int bs_shift,
     int window, float scale_log2, int num_splits, int head_chunks, DecodeFusedArgs fa,
-    const int* __restrict__ live_items, int waves_wanted, const int* __restrict__ step_flags) {
+    const int* __restrict__ live_items, int waves_wanted, const int* __restrict__ step_flags, const float* __restrict__ sink) {
   if constexpr (STREAMED) {
     if (!(step_flags && (step_flags[0] & 1))) {
       attention_decode_body<D, FUSED, DEPTH, true>(q, k_cache, v_cache, item_ctx, block_table, table_width, part_o, part_ml, out, nh,
                                                    nkv, bs_shift, window, scale_log2, num_splits, head_chunks, fa, live_items,
-                                                   waves_wanted);
+                                                   waves_wanted, sink);
       return;
     }
   }
   attention_decode_body<D, FUSED, DEPTH, false>(q, k_cache, v_cache, item_ctx, block_table, table_width, part_o, part_ml, out, nh, nkv,
-                                                bs_shift, window, scale_log2, num_splits, head_chunks, fa, live_items, waves_wanted);
+                                                bs_shift, window, scale_log2, num_splits, head_chunks, fa, live_items, waves_wanted,
+                                                sink);
 }
 
 // out[item, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s. One block of 256 threads per
@@ -470,7 +477,8 @@ __global__ __launch_bounds__(DECODE_BLOCK_WAVES(D) * 64) void attention_decode_k
 #define ME_MAX_SPLITS 1024
 __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const float* __restrict__ part_o,
                                                                        const float* __restrict__ part_ml,
-                                                                       bf16_t* __restrict__ out, int num_splits, int d) {
+                                                                       bf16_t* __restrict__ out, int num_splits, int d,
+                                                                       const float* __restrict__ sink, int nh) {
   __shared__ float wgt[ME_MAX_SPLITS];
   __shared__ float red_max[4], red_sum[4];
   __shared__ float4_t partial[256];
@@ -498,6 +506,8 @@ __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const flo
   if (lane == 0) red_max[wave] = big;
   __syncthreads();
   big = fmaxf(fmaxf(red_max[0], red_max[1]), fmaxf(red_max[2], red_max[3]));
+  const float s2 = sink ? sink[unit % nh] * LOG2E : -INFINITY;  // a sink counts as one more split of weight 1 and no value
+  big = fmaxf(big, s2);
   float part_denom = 0.f;
   for (int s = tid; s < num_splits; s += 256) {
     const float l = ml[s * 2 + 1];
@@ -508,7 +518,7 @@ __global__ __launch_bounds__(256) void attention_decode_combine_kernel(const flo
   part_denom = wave_sum(part_denom);
   if (lane == 0) red_sum[wave] = part_denom;
   __syncthreads();
-  const float denom = (red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]);
+  const float denom = (red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]) + (sink ? fast_exp2(s2 - big) : 0.f);
 
   float4_t accv = {0.f, 0.f, 0.f, 0.f};
   if (grp < groups) {
@@ -552,7 +562,7 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
                           int width, float* part_o, float* part_ml, int items, int nh, int nkv, int bs, int window,
                           float scale_log2, int depth, int num_splits, int block_waves, bf16_t* out,
                           const DecodeFusedArgs* fused, const int* live_items, int waves_wanted, int streamed,
-                          const int* step_flags, int keep_first, hipStream_t stream) {
+                          const int* step_flags, int keep_first, const float* sink, hipStream_t stream) {
   DecodeFusedArgs unfused{};
   unfused.keep_first = keep_first;
   const int chunks = (nh / nkv + 15) / 16;
@@ -564,7 +574,7 @@ static void launch_decode(const bf16_t* q, const bf16_t* kc, const bf16_t* vc, c
 #define ME_DECODE_LAUNCH_AS(FUSED, DEPTH, STREAMED, ARGS)                                                                  \
   attention_decode_kernel<D, FUSED, DEPTH, STREAMED><<<grid, 64 * block_waves, lds, stream>>>(                             \
       q, kc, vc, item_ctx, table, width, part_o, part_ml, out, nh, nkv, bs_shift, window, scale_log2, num_splits, chunks,  \
-      ARGS, live_items, waves_wanted, step_flags)
+      ARGS, live_items, waves_wanted, step_flags, sink)
 #define ME_DECODE_LAUNCH(FUSED, DEPTH, ARGS)                \
   do {                                                      \
     if (streamed)                                           \
@@ -646,7 +656,8 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
                          int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
-                         int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first = 0);
+                         int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first = 0,
+                         const float* sink = nullptr);
 
 // As me_attention_decode_bf16, with the first `keep_first` keys of every item visible behind the window.
 extern "C" int me_attention_decode_bf16_kept(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
@@ -658,6 +669,18 @@ extern "C" int me_attention_decode_bf16_kept(const void* q, const void* k_cache,
   return decode_common(q, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
                        bs, window, scale, split_keys, num_splits, max_ctx, nullptr, live_items, full_splits, waves_wanted,
                        step_flags, stream, keep_first);
+}
+
+// As me_attention_decode_bf16, with a learned logit per head (sink float32 [nh], not multiplied by the scale) that counts once
+// in the softmax's denominator and has no value.
+extern "C" int me_attention_decode_bf16_sink(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
+                                             const int* block_table, int table_width, void* out, float* part_o,
+                                             float* part_ml, int items, int nh, int nkv, int d, int bs, const float* sink,
+                                             float scale, int split_keys, int num_splits, int max_ctx, const int* live_items,
+                                             int full_splits, int waves_wanted, const int* step_flags, hipStream_t stream) {
+  return decode_common(q, k_cache, v_cache, item_ctx, block_table, table_width, out, part_o, part_ml, items, nh, nkv, d,
+                       bs, 0, scale, split_keys, num_splits, max_ctx, nullptr, live_items, full_splits, waves_wanted,
+                       step_flags, stream, 0, sink);
 }
 
 extern "C" int me_attention_decode_bf16(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
@@ -708,7 +731,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
                          const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
                          int nh, int nkv, int d, int bs, int window, float scale, int split_keys, int num_splits,
                          int max_ctx, const DecodeFusedArgs* fused, const int* live_items, int full_splits,
-                         int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first) {
+                         int waves_wanted, const int* step_flags, hipStream_t stream, int keep_first, const float* sink) {
   if (items <= 0) return 0;
   if (keep_first < 0 || (keep_first > 0 && (window <= 0 || fused)))
     return me_fail("me_attention_decode_bf16: keep_first=%d needs a window and the unfused form", keep_first);
@@ -733,6 +756,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   const int block_waves = decode_block_waves(items, nh, nkv, d, num_splits);
   if (!out && block_waves > 1)
     return me_fail("me_attention_decode_bf16: a launch whose blocks add up their splits themselves needs `out`");
+  if (!out && sink) return me_fail("me_attention_decode_bf16: the product that adds up the splits itself knows no sink");
   const int cus = decode_compute_units();
   const long long blocks = (long long)items * nkv * ((nh / nkv + 15) / 16);
   // Keys and values pass through once: loaded as non-temporal they arrive faster where the launch streams hundreds of
@@ -749,7 +773,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   case DD:                                                                                                      \
     launch_decode<DD>(qq, kc, vc, item_ctx, block_table, table_width, part_o, part_ml, items, nh, nkv, bs, window, sl, \
                       depth, num_splits, block_waves, (bf16_t*)out, fused, live_items, waves_wanted, streamed, step_flags, \
-                      keep_first, stream);                                                                      \
+                      keep_first, sink, stream);                                                                \
     break;
   switch (d) {
     ME_DECODE_CASE(32)
@@ -763,7 +787,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   if (me_check_launch("me_attention_decode_bf16")) return 1;
   if (block_waves > 1) return 0;  // the blocks held all splits of their heads and wrote the output themselves
   if (!out) return 0;             // the caller adds up the splits (me_attention_out_product_bf16)
-  attention_decode_combine_kernel<<<items * nh, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, num_splits, d);
+  attention_decode_combine_kernel<<<items * nh, 256, 0, stream>>>(part_o, part_ml, (bf16_t*)out, num_splits, d, sink, nh);
   return me_check_launch("me_attention_decode_combine");
 }
 
@@ -1033,7 +1057,8 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const PrefillWork* __restrict__ work, const int* __restrict__ bundle_first, const int* __restrict__ block_table,
     int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks,
-    int nh, int nkv, int bs_shift, int window, float scale_log2, int tokens_per_block, int keep_first) {
+    int nh, int nkv, int bs_shift, int window, float scale_log2, int tokens_per_block, int keep_first,
+    const float* __restrict__ sink) {
   constexpr int THREADS = WAVES * 64;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   bf16_t* lds = reinterpret_cast<bf16_t*>(lds_raw);
@@ -1139,7 +1164,12 @@ __global__ __launch_bounds__(WAVES * 64) void attention_prefill_kernel(
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       if (!col_ok[nb]) continue;
-      const float inv = 1.f / lsum[nb];
+      float inv = 1.f / lsum[nb];
+      if (sink) {  // one more term exp(sink) in the denominator, with no value (statistics are in units of log2)
+        const float s2 = sink[head[nb]] * LOG2E, top = fmaxf(m[nb], s2);
+        const float keep = fast_exp2(m[nb] - top);
+        inv = keep / (lsum[nb] * keep + fast_exp2(s2 - top));
+      }
       bf16_t* orow = out + ((size_t)tok[nb] * nh + head[nb]) * D;
 #pragma unroll
       for (int dt = 0; dt < D / 16; ++dt) {
@@ -1161,7 +1191,7 @@ __global__ __launch_bounds__(256) void attention_prefill_combine_kernel(const fl
                                                                         const float* __restrict__ part_ml,
                                                                         const int* __restrict__ token_chunks,
                                                                         bf16_t* __restrict__ out, int nh, int d,
-                                                                        int max_chunks) {
+                                                                        int max_chunks, const float* __restrict__ sink) {
   const int tok = blockIdx.x;
   const int nc = token_chunks[tok];
   if (nc <= 1) return;
@@ -1174,7 +1204,9 @@ __global__ __launch_bounds__(256) void attention_prefill_combine_kernel(const fl
     float big = -INFINITY;
     for (int c = 0; c < nc; ++c)
       if (ml[c * 2 + 1] > 0.f) big = fmaxf(big, ml[c * 2]);
-    float denom = 0.f;
+    const float s2 = sink ? sink[head] * LOG2E : -INFINITY;  // a sink counts as one more range of weight 1 and no value
+    big = fmaxf(big, s2);
+    float denom = sink ? fast_exp2(s2 - big) : 0.f;
     float4_t total = {0.f, 0.f, 0.f, 0.f};
     for (int c = 0; c < nc; ++c) {
       const float l = ml[c * 2 + 1];
@@ -1207,7 +1239,7 @@ template <int D, int NB>
 static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf16_t* vc, const PrefillWork* work,
                           const int* bundle_first, const int* table, int width, bf16_t* out,
                           float* part_o, float* part_ml, int max_chunks, int nh, int nkv, int bs_shift, int window,
-                          float sl, int tpb, int keep_first, hipStream_t stream) {
+                          float sl, int tpb, int keep_first, const float* sink, hipStream_t stream) {
   static bool configured = false;  // raise the dynamic LDS limit of this instantiation once
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attention_prefill_kernel<D, NB, PF_WAVES>),
@@ -1218,7 +1250,7 @@ static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf
   }
   attention_prefill_kernel<D, NB, PF_WAVES><<<grid, PF_WAVES * 64, PrefillLds<D>::BYTES, stream>>>(
       q, kc, vc, work, bundle_first, table, width, out, part_o, part_ml, max_chunks, nh, nkv, bs_shift, window, sl, tpb,
-      keep_first);
+      keep_first, sink);
   return 0;
 }
 
@@ -1232,12 +1264,14 @@ static int launch_prefill(dim3 grid, const bf16_t* q, const bf16_t* kc, const bf
 // chunks each token's tile has (1: in one piece).
 // keep_first: with a window, the keys 0 .. keep_first-1 stay visible behind it; the work list then gives a tile whose
 // window has left them behind an entry of its own for them (so such a tile always has chunks).
-extern "C" int me_attention_prefill_bf16_kept(const void* q, const void* k_cache, const void* v_cache, int num_items,
-                                              const int* block_table, int table_width, void* out, const int* work,
-                                              const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
-                                              const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
-                                              int d, int bs, int window, int keep_first, float scale, int columns,
-                                              hipStream_t stream) {
+// sink (float32 [nh] or null): a learned logit per head, not multiplied by the scale, that counts once in the softmax's
+// denominator and has no value.
+static int prefill_common(const void* q, const void* k_cache, const void* v_cache, int num_items,
+                          const int* block_table, int table_width, void* out, const int* work,
+                          const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
+                          const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
+                          int d, int bs, int window, int keep_first, float scale, int columns, const float* sink,
+                          hipStream_t stream) {
   const int num_work = num_bundles;
   if (keep_first < 0 || (keep_first > 0 && window <= 0))
     return me_fail("me_attention_prefill_bf16: keep_first=%d needs a window", keep_first);
@@ -1268,10 +1302,10 @@ extern "C" int me_attention_prefill_bf16_kept(const void* q, const void* k_cache
   case DD:                                                                                                         \
     rc = wide ? launch_prefill<DD, 2>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table,       \
                                       table_width, (bf16_t*)out, part_o, part_ml, max_chunks, nh, nkv, bs_shift,   \
-                                      window, sl, tpb, keep_first, stream)                                         \
+                                      window, sl, tpb, keep_first, sink, stream)                                   \
               : launch_prefill<DD, 1>(grid, qq, kc, vc, (const PrefillWork*)work, bundle_first, block_table,       \
                                       table_width, (bf16_t*)out, part_o, part_ml, max_chunks, nh, nkv, bs_shift,   \
-                                      window, sl, tpb, keep_first, stream);                                        \
+                                      window, sl, tpb, keep_first, sink, stream);                                  \
     break;
   switch (d) {
     ME_PREFILL_CASE(32)
@@ -1286,10 +1320,31 @@ extern "C" int me_attention_prefill_bf16_kept(const void* q, const void* k_cache
   if (me_check_launch("me_attention_prefill_bf16")) return 1;
   if (max_chunks > 1) {
     attention_prefill_combine_kernel<<<num_tokens, 256, 0, stream>>>(part_o, part_ml, token_chunks, (bf16_t*)out, nh, d,
-                                                                     max_chunks);
+                                                                     max_chunks, sink);
     return me_check_launch("me_attention_prefill_combine");
   }
   return 0;
+}
+
+extern "C" int me_attention_prefill_bf16_kept(const void* q, const void* k_cache, const void* v_cache, int num_items,
+                                              const int* block_table, int table_width, void* out, const int* work,
+                                              const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
+                                              const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
+                                              int d, int bs, int window, int keep_first, float scale, int columns,
+                                              hipStream_t stream) {
+  return prefill_common(q, k_cache, v_cache, num_items, block_table, table_width, out, work, bundle_first, num_bundles, part_o,
+                        part_ml, token_chunks, max_chunks, num_tokens, nh, nkv, d, bs, window, keep_first, scale, columns, nullptr,
+                        stream);
+}
+
+// All keys visible, with a sink (see prefill_common).
+extern "C" int me_attention_prefill_bf16_sink(const void* q, const void* k_cache, const void* v_cache, int num_items,
+                                              const int* block_table, int table_width, void* out, const int* work,
+                                              const int* bundle_first, int num_bundles, float* part_o, float* part_ml,
+                                              const int* token_chunks, int max_chunks, int num_tokens, int nh, int nkv,
+                                              int d, int bs, const float* sink, float scale, int columns, hipStream_t stream) {
+  return prefill_common(q, k_cache, v_cache, num_items, block_table, table_width, out, work, bundle_first, num_bundles, part_o,
+                        part_ml, token_chunks, max_chunks, num_tokens, nh, nkv, d, bs, 0, 0, scale, columns, sink, stream);
 }
 
 extern "C" int me_attention_prefill_bf16(const void* q, const void* k_cache, const void* v_cache, int num_items,

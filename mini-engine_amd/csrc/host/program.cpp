@@ -143,6 +143,15 @@ bool attention_is_plain(const Op& op) {
   return (op.i[9] == 0 || op.i[9] == op.i[2]) && op.i[10] == 0 && op.i[11] == 0 && op.i[12] == 0 && op.i[13] == 0 && op.i[14] == 0;
 }
 
+// A latent attention operation: the rows of its value pages (i8; 0: the latent's rank), and whether the matrix-core attention
+// kernels serve it: bfloat16, value pages that hold the whole key (the kernels take keys and values of one size), a key
+// size they are built for, at most 16 heads (all of them share the one key/value head).
+int latent_value_rows(const Op& op) { return op.i[8] ? (int)op.i[8] : (int)op.i[3]; }
+bool latent_takes_matrix_cores(const Op& op, int dtype) {
+  const int dk = (int)(op.i[3] + op.i[2]);
+  return dtype == kBF16 && latent_value_rows(op) == dk && me_attention_mfma_supported(dk, (int)op.i[5]) && op.i[0] <= 16;
+}
+
 // How many residual streams the tokens of a program have (kOpStreams; 1 without).
 int streams_of(const std::vector<Op>& ops) {
   int s = 1;
@@ -665,18 +674,44 @@ class Run {
     const long long row = (long long)nh * (d + r) + dk + nh;
     if (values_[op.in].cols != row) throw Error(kBadValue, "the projections of a latent attention layer have the wrong width");
     const int32_t* table = idx(s_.lay.tables[g]);
-    const int width = s_.lay.widths[g];
+    const int width = s_.lay.widths[g], items = s_.lay.items;
+    const int vr = latent_value_rows(op);  // rows of a value page: the latent's, or the whole key's for the matrix-core kernels
+    const float* sink = (const float*)op.p[6];
+    const float scale = op.f[1];
     const char* proj = (const char*)bufs_[op.in];
     void* qa = arena_.take((size_t)t_ * nh * dk * elem_);
-    void* ol = arena_.take((size_t)t_ * nh * rank * elem_);
+    void* ol = arena_.take((size_t)t_ * nh * vr * elem_);
+    const void *kc = op.p[2], *vc = op.p[3];
     ok(me_latent_prepare(proj, row, (const float*)op.p[0], (const float*)op.p[1], idx(s_.lay.positions), idx(s_.lay.token_item), table,
-                         width, qa, (void*)op.p[2], (void*)op.p[3], t_, nh, d, r, rank, rank, bs, op.f[0], dtype_, stream_));
+                         width, qa, (void*)kc, (void*)vc, t_, nh, d, r, rank, vr, bs, op.f[0], dtype_, stream_));
     ok(me_head_product(proj, row, d + r, op.p[4], qa, (long long)nh * dk, dk, nullptr, 0, t_, nh, rank, d, dtype_, stream_));
-    ok(me_attention_general_gated(qa, op.p[2], op.p[3], idx(s_.lay.positions), idx(s_.lay.token_item), table, width, ol, t_, nh, 1, dk,
-                                  rank, bs, 0, 0, nullptr, 0, op.f[1], (const float*)op.p[6], nullptr, 0, dtype_, s_.lay.items,
-                                  stream_));
-    ok(me_head_product(ol, (long long)nh * rank, rank, op.p[5], bufs_[op.out], (long long)nh * dv, dv,
-                       proj + (size_t)(row - nh) * elem_, row, t_, nh, dv, rank, dtype_, stream_));
+    if (latent_takes_matrix_cores(op, dtype_) && s_.decode_only) {
+      // one new token per item: the split-context kernel; all heads share the one key/value head, 16 to a wave
+      if ((long long)width * bs < s_.max_ctx) throw Error(kBadValue, "the block table cannot hold the step's longest context");
+      const SplitPlan sp = split_plan(items, (nh + 15) / 16, s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
+      float* part_o = (float*)arena_.take((size_t)items * nh * sp.num_splits * dk * 4);
+      float* part_ml = (float*)arena_.take((size_t)items * nh * sp.num_splits * 2 * 4);
+      ok(me_attention_decode_bf16_sink(qa, kc, vc, idx(s_.lay.item_ctx), table, width, ol, part_o, part_ml, items, nh, 1, dk, bs, sink,
+                                       scale, sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves,
+                                       idx(s_.lay.live_items) + 1, stream_));
+    } else if (latent_takes_matrix_cores(op, dtype_)) {
+      auto it = s_.plans.find({nh, 1, dk, 0, 0});
+      if (it == s_.plans.end()) throw Error(kBroken, "the step has no work list for a latent attention layer");
+      const StepView::Plan& p = it->second;
+      float *part_o = nullptr, *part_ml = nullptr;
+      if (p.max_chunks > 1) {
+        part_o = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * dk * 4);
+        part_ml = (float*)arena_.take((size_t)t_ * nh * p.max_chunks * 2 * 4);
+      }
+      ok(me_attention_prefill_bf16_sink(qa, kc, vc, items, table, width, ol, idx(p.work), idx(p.bundle_first), p.bundles, part_o, part_ml,
+                                        p.token_chunks >= 0 ? idx(p.token_chunks) : nullptr, p.max_chunks, t_, nh, 1, dk, bs, sink, scale,
+                                        p.columns, stream_));
+    } else {
+      ok(me_attention_general_gated(qa, kc, vc, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, ol, t_, nh, 1, dk, vr, bs,
+                                    0, 0, nullptr, 0, scale, sink, nullptr, 0, dtype_, items, stream_));
+    }
+    ok(me_head_product(ol, (long long)nh * vr, vr, op.p[5], bufs_[op.out], (long long)nh * dv, dv, proj + (size_t)(row - nh) * elem_, row,
+                       t_, nh, dv, rank, dtype_, stream_));
   }
 
   // A feed-forward of routed experts (csrc/routed_ff.hip): its result waits as one partial sum per expert of a token.
@@ -795,6 +830,10 @@ std::vector<std::vector<int>> Program::prefill_geometries() const {
   std::vector<std::vector<int>> out;
   if (dtype_ != kBF16) return out;
   for (const Op& op : ops_) {
+    if (op.kind == kOpLatentAttention && latent_takes_matrix_cores(op, dtype_)) {
+      std::vector<int> key = {(int)op.i[0], 1, (int)(op.i[3] + op.i[2]), 0, 0};
+      if (std::find(out.begin(), out.end(), key) == out.end()) out.push_back(key);
+    }
     if (op.kind != kOpAttention) continue;
     const int nh = (int)op.i[0], nkv = (int)op.i[1], d = (int)op.i[2], bs = (int)op.i[4], window = (int)op.i[5];
     if (!attention_is_plain(op) && !attention_takes_tiled_prefill(op, dtype_)) continue;
@@ -818,8 +857,21 @@ size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t 
       need = std::max<size_t>((size_t)kMaxRuns * std::min<int64_t>(tokens, kSmallMaxRows), (size_t)tokens) * op.i[0] * 4 + pad;
     if (op.kind == kOpDecayState)
       need = (size_t)me_decay_state_workspace(tokens, items, (int)op.i[0], (int)op.i[1], (int)op.i[2]) + pad;
-    if (op.kind == kOpLatentAttention)
-      need = (size_t)tokens * op.i[0] * (2 * op.i[3] + op.i[2]) * elem + 2 * pad;
+    if (op.kind == kOpLatentAttention) {
+      const int nh = (int)op.i[0], dk = (int)(op.i[3] + op.i[2]);
+      need = (size_t)tokens * nh * 2 * dk * elem + 2 * pad;
+      if (latent_takes_matrix_cores(op, dtype_)) {  // the splits' partial results of a decode step, or those of cut tiles
+        size_t most = 0;
+        for (int64_t b = 1; b <= items; ++b) {
+          int keys, splits;
+          decode_splits((int)std::max<int64_t>(1, (b + 1) / 2), (nh + 15) / 16, (int)max_ctx, keys, splits);
+          most = std::max(most, (size_t)b * splits);
+        }
+        const size_t decode = most * nh * (dk + 2) * 4 + 2 * pad;
+        const size_t prefill = (size_t)(256ll << 20) + (size_t)(256ll << 20) * 2 / dk + (size_t)tokens * nh * 8 + 2 * pad;
+        need += std::max(decode, tokens > items ? prefill : (size_t)0);
+      }
+    }
     if (op.kind == kOpRoutedFF)
       need = (size_t)op.i[1] * tokens * hidden_ * 4 + (size_t)me_routed_ff_workspace(tokens, (int)op.i[0], (int)op.i[1], (int)op.i[2], (int)elem) +
              2 * pad;

@@ -60,7 +60,8 @@ enum OpKind {
                       // key part, a gate per head); p0 weight of the latent's norm, p1 rotary table [positions, 2, r/2], p2 key
                       // pages [page, 1, slot, rank + r], p3 value pages [page, 1, rank, slot], p4 the keys' map per head, transposed
                       // [heads, rank, d], p5 the values' map per head [heads, dv, rank], p6 sink float32 [heads] or null;
-                      // i0 heads, i1 d, i2 r, i3 rank, i4 dv, i5 page size, i6 cache group, i7 positions the table covers;
+                      // i0 heads, i1 d, i2 r, i3 rank, i4 dv, i5 page size, i6 cache group, i7 positions the table covers,
+                      // i8 rows of a value page (0: rank; rank + r: the whole key, as the matrix-core kernels want it);
                       // f0 eps, f1 scale -> out [tokens, heads * dv]
   kOpRoutedFF = 18,   // in: normed activations; p0 router W float32 [E, hidden], p1 experts' gate and up rows [E, 2 ff, hidden],
                       // p2 experts' down rows [E, hidden, ff]; i0 E, i1 experts a token, i2 ff, i3 code of the activation

@@ -115,6 +115,15 @@ int me_routed_ff_max_tiles(long long tokens, int E, int top);
 long long me_routed_ff_workspace(long long tokens, int E, int top, int ff, int elem);
 int me_routed_ff(const void* h, const float* Wr, const void* W_gu, const void* W_down, float* parts, void* workspace, int num_tokens,
                  int hidden, int E, int top, int ff, int act, int dtype, hipStream_t stream);
+int me_attention_decode_bf16_sink(const void* q, const void* k_cache, const void* v_cache, const int* item_ctx,
+                                  const int* block_table, int table_width, void* out, float* part_o, float* part_ml, int items,
+                                  int nh, int nkv, int d, int bs, const float* sink, float scale, int split_keys, int num_splits,
+                                  int max_ctx, const int* live_items, int full_splits, int waves_wanted, const int* step_flags,
+                                  hipStream_t stream);
+int me_attention_prefill_bf16_sink(const void* q, const void* k_cache, const void* v_cache, int num_items, const int* block_table,
+                                   int table_width, void* out, const int* work, const int* bundle_first, int num_bundles,
+                                   float* part_o, float* part_ml, const int* token_chunks, int max_chunks, int num_tokens, int nh,
+                                   int nkv, int d, int bs, const float* sink, float scale, int columns, hipStream_t stream);
 int me_unturn_rows(void* rows, const float* table, int pairing, const int* positions, int num_tokens, int heads, int n,
                    int dtype, hipStream_t stream);
 int me_gemm_f32(const float* A, const float* W, float* C, int M, int N, int K, hipStream_t stream);

@@ -334,11 +334,13 @@ class StepProgram:
         self._want(value_map, self.dtype, (heads, value_dim, rank), "the values' map")
         if sink is not None:
             self._want(sink, torch.float32, (heads,), "sink")
-        if tuple(k_cache.shape[1:]) != (1, block_size, rank + rotary_dim) or tuple(v_cache.shape[1:]) != (1, rank, block_size):
-            raise ValueError("a latent attention layer keeps pages of one head: keys of rank + rotary_dim, values of rank elements")
+        value_rows = int(v_cache.shape[2])  # the latent's rank, or the whole key's size (what the matrix-core kernels take)
+        if (tuple(k_cache.shape[1:]) != (1, block_size, rank + rotary_dim) or tuple(v_cache.shape[1:]) != (1, value_rows, block_size)
+                or value_rows not in (rank, rank + rotary_dim)):
+            raise ValueError("a latent attention layer keeps pages of one head: keys of rank + rotary_dim, values of rank (or as many) elements")
         out = self.take(heads * value_dim)
         self.op(LATENT_ATTENTION, in_=proj, out=out, ptrs=[latent_norm, rope, k_cache, v_cache, key_map, value_map, sink],
-                ints=[heads, head_dim, rotary_dim, rank, value_dim, block_size, group, rope.shape[0]], floats=[eps, scale])
+                ints=[heads, head_dim, rotary_dim, rank, value_dim, block_size, group, rope.shape[0], value_rows], floats=[eps, scale])
         return out
 
     def routed_ff(self, x: int, *, router: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, top_k: int, activation: str) -> None:

@@ -21,6 +21,7 @@ from ..weights.loader import TensorWant
 from .base import MIXERS, POSITION_ENCODINGS, KVBinding, KVCacheNeed, Mixer
 
 MAX_KEY_DIM = 256  # what the attention kernel that takes every size allows for rank + rotary_dim
+MATRIX_CORE_KEY_DIMS = (32, 64, 96, 128, 192, 256)  # csrc/attention_mfma.hip: me_attention_mfma_supported
 
 
 class LatentAttention(Mixer):
@@ -75,7 +76,11 @@ class LatentAttention(Mixer):
 
     # ---- cache
     def cache_need(self):
-        return KVCacheNeed(1, self.rank + self.r, 0, value_dim=self.rank)
+        # bfloat16 with a key size that the matrix-core attention kernels take and at most 16 heads: those kernels read keys and
+        # values of one size, so the value pages hold the whole key (its first `rank` rows are the values that count)
+        dk = self.rank + self.r
+        whole = self.dtype is torch.bfloat16 and dk in MATRIX_CORE_KEY_DIMS and self.nh <= 16
+        return KVCacheNeed(1, dk, 0, value_dim=dk if whole else self.rank)
 
     # ---- step
     def forward(self, h, batch, cache=None):

@@ -64,10 +64,15 @@ def configs() -> dict[str, dict]:
         "D": model(211, 64, 0, 1e-4, [
             latent(2, 16, 16, 16, 32, 0.2, 1e3, mlp=dense(72)),
             attention(4, 2, 16, 16, 0.25, q_temp=(0.3, 16), mlp=moe(4, 2, 32))]),
+        # sizes that the matrix-core attention kernels take in bfloat16: keys and values of 64 elements; a latent key of
+        # 96 + 32 elements under 16 heads
+        "E": model(260, 128, 2, 1e-6, [
+            attention(8, 2, 64, 64, 0.125, q_temp=(0.3, 40), mlp=dense(160)),
+            latent(16, 24, 32, 16, 96, 0.13, 1e4, scaling=(4.0, 128, 16.0, 1.0), mlp=moe(6, 2, 64))]),
     }
 
 
-BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16}
+BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16}
 
 
 def wants_of(cfg: dict):
