@@ -368,11 +368,36 @@ def gonurax_config(size: str):
                                     "norm": {"eps": 1e-6, "groups": 2}, "layers": order})
 
 
+def kifezen_config(size: str):
+    """Eight layers over two residual streams: six of attention over cached latents (16 heads of 128 + 64 rotated, values of
+    128, a latent of 192, so a cached key of 256 elements), two of grouped-query attention (heads of 128, 8 key/value heads, a
+    temperature on the queries); dense feed-forwards of the size's width in turns with 16 routed experts of half that width,
+    two of them a token (as many weights at work per token as in the dense ones, eight times as many in all)."""
+    from mini_engine_amd.models.kifezen import KifezenConfig
+
+    z = DESIGN_SIZES[size]
+    h = z["heads"]
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 2}, "router": {"experts": 16, "top": 2}}
+    rot = {"base": 1e4, "dims": 64, "scaling": {"factor": 40.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    lat = {"heads": h, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5, "rot": rot}
+    att = {"heads": h, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "q_temp": {"coef": 0.1, "every": 1024}}
+    order = [{"type": "latent_attention", "mixer": lat, "mlp": dense}, {"type": "latent_attention", "mixer": lat, "mlp": moe},
+             {"type": "attention", "mixer": att, "mlp": dense}, {"type": "latent_attention", "mixer": lat, "mlp": moe}] * (DESIGN_LAYERS // 4)
+    return KifezenConfig.from_dict({"architecture": "Kifezen", "vocab": DESIGN_VOCAB, "width": z["width"], "streams": 2,
+                                    "norm": {"eps": 1e-6}, "layers": order})
+
+
+DESIGNS = {"gonurax": ("Gonurax", gonurax_config), "kifezen": ("Kifezen", kifezen_config)}
+
+
 def design_line(args) -> dict:
-    """Prefill and decode throughput of the Gonurax design beside the Qwen3 dense design at equal layer sizes (random
+    """Prefill and decode throughput of a design (Gonurax, Kifezen) beside the Qwen3 dense design at equal layer sizes (random
     weights, eight layers): a 2,048-token prompt, and decode steps at batch 1, 8 and 64 behind a context of 2,304."""
     from mini_engine_amd.models.qwen3 import Qwen3Config
 
+    design = args.design
+    arch_name, config_of = DESIGNS[design]
     ctx, out = 2304, {}
     sizes = [z for z in args.design_sizes.split(",") if z]
     for size in sizes:
@@ -380,7 +405,9 @@ def design_line(args) -> dict:
         qwen = Qwen3Config(vocab_size=DESIGN_VOCAB, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6, num_hidden_layers=DESIGN_LAYERS,
                            hidden_size=z["width"], num_attention_heads=z["heads"], num_key_value_heads=8,
                            intermediate_size=z["ff"], tie_word_embeddings=True, max_position_embeddings=40960)
-        for name, arch, cfg in (("gonurax", "Gonurax", gonurax_config(size)), ("qwen3", "Qwen3ForCausalLM", qwen)):
+        for name, arch, cfg in ((design, arch_name, config_of(size)), ("qwen3", "Qwen3ForCausalLM", qwen)):
+            if args.design_alone and name == "qwen3":
+                continue
             bench = DecodeBench(cfg, args.dtype, ctx, 64, architecture=arch)
             pf = bench.prefill(args.prefill_tokens)
             out[f"{name}_{size}_prefill_{pf['tokens']}_tok_s"] = pf["value"]
@@ -393,12 +420,12 @@ def design_line(args) -> dict:
             del bench
             release()
     first = sizes[0]
-    return {"metric": f"decode tok/s at batch 8 (Gonurax design, width {DESIGN_SIZES[first]['width']}, {DESIGN_LAYERS} layers)",
-            "value": out[f"gonurax_{first}_decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-            "warmup": args.warmup, "ms_per_step": out[f"gonurax_{first}_decode_b8_ms_per_step"], "higher_is_better": True,
+    return {"metric": f"decode tok/s at batch 8 ({arch_name} design, width {DESIGN_SIZES[first]['width']}, {DESIGN_LAYERS} layers)",
+            "value": out[f"{design}_{first}_decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": out[f"{design}_{first}_decode_b8_ms_per_step"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights",
-            "config": {"model": "Gonurax design beside the Qwen3 dense design at equal layer sizes", "layers": DESIGN_LAYERS,
+            "config": {"model": f"{arch_name} design beside the Qwen3 dense design at equal layer sizes", "layers": DESIGN_LAYERS,
                        "vocab": DESIGN_VOCAB, "sizes": {z: DESIGN_SIZES[z] for z in sizes}, "seq_len": ctx, "global_batch": 8,
                        "parallelism": "single GPU"},
             "points": out}
@@ -418,9 +445,10 @@ def main() -> int:
     ap.add_argument("--skip-prefill", action="store_true", help="profiling aid: do not measure the prefill")
     ap.add_argument("--skip-extras", action="store_true",
                     help="profiling aid: only the decode steps and the prefill (no serving workloads, no float32 point, no probes)")
-    ap.add_argument("--design", default="", choices=["", "gonurax"],
+    ap.add_argument("--design", default="", choices=["", "gonurax", "kifezen"],
                     help="instead of the default workload: this design beside the Qwen3 dense design at equal layer sizes")
     ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design to measure, comma separated")
+    ap.add_argument("--design-alone", action="store_true", help="profiling aid: --design without the Qwen3 model beside it")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine runs on one GPU)")

@@ -671,8 +671,9 @@ class Run {
     if (op.i[7] < s_.max_ctx)
       throw Error(kBadValue, "the rotary table covers " + std::to_string(op.i[7]) + " positions, the step may reach " +
                                  std::to_string(s_.max_ctx));
-    const long long row = (long long)nh * (d + r) + dk + nh;
-    if (values_[op.in].cols != row) throw Error(kBadValue, "the projections of a latent attention layer have the wrong width");
+    // (the rows may be padded behind the gates, so that every row starts at a multiple of 16 bytes)
+    const long long used = (long long)nh * (d + r) + dk + nh, row = values_[op.in].cols;
+    if (row < used) throw Error(kBadValue, "the projections of a latent attention layer have the wrong width");
     const int32_t* table = idx(s_.lay.tables[g]);
     const int width = s_.lay.widths[g], items = s_.lay.items;
     const int vr = latent_value_rows(op);  // rows of a value page: the latent's, or the whole key's for the matrix-core kernels
@@ -710,7 +711,7 @@ class Run {
       ok(me_attention_general_gated(qa, kc, vc, idx(s_.lay.positions), idx(s_.lay.token_item), table, width, ol, t_, nh, 1, dk, vr, bs,
                                     0, 0, nullptr, 0, scale, sink, nullptr, 0, dtype_, items, stream_));
     }
-    ok(me_head_product(ol, (long long)nh * vr, vr, op.p[5], bufs_[op.out], (long long)nh * dv, dv, proj + (size_t)(row - nh) * elem_, row,
+    ok(me_head_product(ol, (long long)nh * vr, vr, op.p[5], bufs_[op.out], (long long)nh * dv, dv, proj + (size_t)(used - nh) * elem_, row,
                        t_, nh, dv, rank, dtype_, stream_));
   }
 

@@ -109,6 +109,38 @@ __global__ __launch_bounds__(256) void head_product_kernel(const T* __restrict__
   }
 }
 
+// The same on the matrix cores (bfloat16; k and all strides multiples of 8 elements, bases at multiples of 16 bytes): a block
+// takes 16 * MT tokens and 64 columns of a head, a wave 16 columns (tile_product.h: wave_product_bf16).
+template <int MT>
+__global__ __launch_bounds__(256) void head_product_mfma_kernel(const bf16_t* __restrict__ x, size_t x_row, size_t x_head,
+                                                                const bf16_t* __restrict__ W, bf16_t* __restrict__ out, size_t out_row,
+                                                                size_t out_head, const bf16_t* __restrict__ gate, size_t gate_row,
+                                                                int num_tokens, int n, int k) {
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1), r = lane & 15, g = lane >> 4;
+  const int t0 = blockIdx.x * 16 * MT, n0 = blockIdx.y * 64 + wave * 16, h = blockIdx.z;
+  if (n0 >= n) return;
+  const bf16_t* wrow[1] = {n0 + r < n ? W + ((size_t)h * n + n0 + r) * k : nullptr};
+  const bf16_t* xrow[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int tok = t0 + t * 16 + r;
+    xrow[t] = tok < num_tokens ? x + (size_t)tok * x_row + (size_t)h * x_head : nullptr;
+  }
+  tp_float4 acc[MT][1];
+  wave_product_bf16<MT, 1>(xrow, wrow, k, acc);
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int tok = t0 + t * 16 + r;
+    if (tok >= num_tokens) continue;
+    const float gv = gate ? 1.f / (1.f + expf(-to_float(gate[(size_t)tok * gate_row + h]))) : 1.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = n0 + 4 * g + i;
+      if (col < n) out[(size_t)tok * out_row + (size_t)h * out_head + col] = from_float<bf16_t>(acc[t][0][i] * gv);
+    }
+  }
+}
+
 extern "C" int me_head_product(const void* x, long long x_row, long long x_head, const void* W, void* out, long long out_row,
                                long long out_head, const void* gate, long long gate_row, int num_tokens, int heads, int n, int k,
                                int dtype, hipStream_t stream) {
@@ -116,6 +148,17 @@ extern "C" int me_head_product(const void* x, long long x_row, long long x_head,
   if (heads <= 0 || heads > 65535 || n <= 0 || k <= 0) return me_fail("me_head_product: heads=%d n=%d k=%d", heads, n, k);
   const dim3 grid((num_tokens + TP_ROWS - 1) / TP_ROWS, (n + TP_COLS - 1) / TP_COLS, heads);
   if (grid.y > 65535) return me_fail("me_head_product: %d columns a head", n);
+  if (dtype == ME_BF16 && k % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 && (((uintptr_t)x | (uintptr_t)W) & 15) == 0) {
+    if (num_tokens >= 64)
+      head_product_mfma_kernel<4><<<dim3((num_tokens + 63) / 64, grid.y, heads), 256, 0, stream>>>(
+          (const bf16_t*)x, (size_t)x_row, (size_t)x_head, (const bf16_t*)W, (bf16_t*)out, (size_t)out_row, (size_t)out_head,
+          (const bf16_t*)gate, (size_t)gate_row, num_tokens, n, k);
+    else
+      head_product_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)x, (size_t)x_row, (size_t)x_head, (const bf16_t*)W,
+                                                            (bf16_t*)out, (size_t)out_row, (size_t)out_head, (const bf16_t*)gate,
+                                                            (size_t)gate_row, num_tokens, n, k);
+    return me_check_launch("me_head_product");
+  }
   if (dtype == ME_F32)
     head_product_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, (size_t)x_row, (size_t)x_head, (const float*)W, (float*)out,
                                                          (size_t)out_row, (size_t)out_head, (const float*)gate, (size_t)gate_row,

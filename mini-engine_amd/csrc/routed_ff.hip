@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256) void routed_route_kernel(const T* __restrict__
 }
 
 // plan: [0] number of tiles; [1 + 3 i ..] tile i: expert, first position, pairs; sorted [P]: the pair at each position.
-__global__ __launch_bounds__(1024) void routed_sort_kernel(const int* __restrict__ ids, int P, int E, int max_tiles,
+__global__ __launch_bounds__(1024) void routed_sort_kernel(const int* __restrict__ ids, int P, int E, int max_tiles, int tile_rows,
                                                            int* __restrict__ plan, int* __restrict__ sorted) {
   __shared__ int count[RF_MAX_EXPERTS], first[RF_MAX_EXPERTS];
   for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
@@ -68,10 +68,10 @@ __global__ __launch_bounds__(1024) void routed_sort_kernel(const int* __restrict
     int at = 0, tiles = 0;
     for (int e = 0; e < E; ++e) {
       first[e] = at;
-      for (int b = 0; b < count[e] && tiles < max_tiles; b += TP_ROWS, ++tiles) {
+      for (int b = 0; b < count[e] && tiles < max_tiles; b += tile_rows, ++tiles) {
         plan[1 + 3 * tiles] = e;
         plan[2 + 3 * tiles] = at + b;
-        plan[3 + 3 * tiles] = min(TP_ROWS, count[e] - b);
+        plan[3 + 3 * tiles] = min(tile_rows, count[e] - b);
       }
       at += count[e];
     }
@@ -133,6 +133,53 @@ __global__ __launch_bounds__(256) void routed_down_kernel(const T* __restrict__ 
   }
 }
 
+// The two products on the matrix cores (bfloat16; hidden and ff multiples of 8): a tile is up to 16 * MT pairs of one expert,
+// a block takes 64 columns of it, a wave 16 (tile_product.h: wave_product_bf16). GATED: rows of h gathered by the pairs'
+// tokens, gate and up rows of the same columns side by side, act(gate) * up -> acts; else rows of acts, the down rows,
+// weight * product -> parts. Tiles of 64 pairs (prompts) read an expert's weights a quarter as often as tiles of 16.
+template <int MT, bool GATED>
+__global__ __launch_bounds__(256) void routed_tile_mfma_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
+                                                               const int* __restrict__ plan, const int* __restrict__ sorted,
+                                                               const float* __restrict__ wts, bf16_t* __restrict__ acts,
+                                                               float* __restrict__ parts, int num_tokens, int N, int K, int top,
+                                                               int act) {
+  const int tile = blockIdx.x;
+  if (tile >= plan[0]) return;
+  const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1), r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.y * 64 + wave * 16;
+  if (n0 >= N) return;
+  constexpr int ACCS = GATED ? 2 : 1;
+  const bf16_t* wrow[ACCS];
+  const bf16_t* w0 = n0 + r < N ? W + ((size_t)e * ACCS * N + n0 + r) * K : nullptr;
+  wrow[0] = w0;
+  if (GATED) wrow[ACCS - 1] = w0 ? w0 + (size_t)N * K : nullptr;
+  const bf16_t* xrow[MT];
+  int pair[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int row = t * 16 + r;
+    pair[t] = row < rows ? sorted[begin + row] : -1;
+    xrow[t] = row < rows ? x + (GATED ? (size_t)(pair[t] / top) : (size_t)(begin + row)) * K : nullptr;
+  }
+  tp_float4 acc[MT][ACCS];
+  wave_product_bf16<MT, ACCS>(xrow, wrow, K, acc);
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    if (pair[t] < 0) continue;
+    const int row = t * 16 + r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = n0 + 4 * g + i;
+      if (col >= N) continue;
+      if (GATED)
+        acts[(size_t)(begin + row) * N + col] = from_float<bf16_t>(gate_act(acc[t][0][i], act) * acc[t][ACCS - 1][i]);
+      else
+        parts[((size_t)(pair[t] % top) * num_tokens + pair[t] / top) * N + col] = wts[pair[t]] * acc[t][0][i];
+    }
+  }
+}
+
 extern "C" int me_routed_ff_max_tiles(long long tokens, int E, int top) {
   return (int)((tokens * top + TP_ROWS - 1) / TP_ROWS) + E;
 }
@@ -162,16 +209,36 @@ extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, co
   const dim3 g_up(max_tiles, (ff + TP_COLS - 1) / TP_COLS), g_down(max_tiles, (hidden + TP_COLS - 1) / TP_COLS);
   if (g_up.y > 65535 || g_down.y > 65535) return me_fail("me_routed_ff: hidden=%d ff=%d", hidden, ff);
   (void)elem;
+  const bool aligned = ((((uintptr_t)h | (uintptr_t)W_gu | (uintptr_t)W_down | (uintptr_t)acts) & 15) == 0);
+  if (dtype == ME_BF16 && hidden % 8 == 0 && ff % 8 == 0 && aligned) {  // the matrix cores
+    const int wide = P >= 32ll * E;  // 32 and more pairs an expert on average: tiles of 64 pairs
+    routed_route_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
+    routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, wide ? 64 : 16, plan, sorted);
+    if (wide) {
+      const unsigned tiles64 = (unsigned)((P + 63) / 64) + E;  // fewer tiles than the list's bound: whole blocks that only return
+      const dim3 g_up(tiles64, (ff + TP_COLS - 1) / TP_COLS), g_down(tiles64, (hidden + TP_COLS - 1) / TP_COLS);
+      routed_tile_mfma_kernel<4, true><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
+                                                                 nullptr, num_tokens, ff, hidden, top, act);
+      routed_tile_mfma_kernel<4, false><<<g_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
+                                                                  parts, num_tokens, hidden, ff, top, act);
+    } else {
+      routed_tile_mfma_kernel<1, true><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
+                                                                 nullptr, num_tokens, ff, hidden, top, act);
+      routed_tile_mfma_kernel<1, false><<<g_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
+                                                                  parts, num_tokens, hidden, ff, top, act);
+    }
+    return me_check_launch("me_routed_ff");
+  }
   if (dtype == ME_F32) {
     routed_route_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)h, Wr, ids, wts, hidden, E, top);
-    routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, plan, sorted);
+    routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, TP_ROWS, plan, sorted);
     routed_gate_up_kernel<float><<<g_up, 256, 0, stream>>>((const float*)h, (const float*)W_gu, plan, sorted, (float*)acts, hidden, ff,
                                                             top, act);
     routed_down_kernel<float><<<g_down, 256, 0, stream>>>((const float*)acts, (const float*)W_down, plan, sorted, wts, parts,
                                                           num_tokens, hidden, ff, top);
   } else {
     routed_route_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
-    routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, plan, sorted);
+    routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, TP_ROWS, plan, sorted);
     routed_gate_up_kernel<bf16_t><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, (bf16_t*)acts, hidden,
                                                              ff, top, act);
     routed_down_kernel<bf16_t><<<g_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, parts,

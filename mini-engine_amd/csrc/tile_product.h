@@ -49,3 +49,47 @@ __device__ __forceinline__ void tile_product(RowPtr row_ptr, int rows, const T* 
     __syncthreads();
   }
 }
+
+// ---------------------------------------------------------------------------------------------------------------------
+// The same product on the matrix cores, bfloat16 operands and float32 sums: 16 * MT rows of x times ACCS tiles of 16 weight
+// rows, by one wave, with v_mfma_f32_16x16x32_bf16 in the transposed arrangement (C^T[n, m] = sum_k W[n, k] X[m, k]): lane l
+// feeds W[n0 + l % 16][k + 8 (l / 16) ..] and X[m0 + l % 16][k + 8 (l / 16) ..], eight elements (16 bytes) each, straight
+// from memory, and receives C[m0 + l % 16][n0 + 4 (l / 16) .. + 4]. k is a multiple of 8 and every row starts at a multiple of
+// 16 bytes (the callers check). Rows do not meet in the arithmetic: a row's sums are the same bits in any tile.
+typedef __bf16 tp_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float tp_float4 __attribute__((ext_vector_type(4)));
+
+// xrow[t]: the row of x that this lane feeds in row tile t (or null: zeros); wrow[a]: its weight row in tile a (or null).
+template <int MT, int ACCS>
+__device__ __forceinline__ void wave_product_bf16(const bf16_t* const (&xrow)[MT], const bf16_t* const (&wrow)[ACCS], int k,
+                                                  tp_float4 (&acc)[MT][ACCS]) {
+  const int g = (threadIdx.x & 63) >> 4;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int a = 0; a < ACCS; ++a) acc[t][a] = (tp_float4){0.f, 0.f, 0.f, 0.f};
+  constexpr int U = 2;  // chunks of 32 whose loads are asked for together
+  for (int k0 = 0; k0 < k; k0 += 32 * U) {
+    tp_bf16x8 wf[U][ACCS], xf[U][MT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int at = k0 + 32 * u + 8 * g;
+#pragma unroll
+      for (int a = 0; a < ACCS; ++a) {
+        wf[u][a] = tp_bf16x8{};
+        if (wrow[a] && at < k) wf[u][a] = *reinterpret_cast<const tp_bf16x8*>(wrow[a] + at);
+      }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        xf[u][t] = tp_bf16x8{};
+        if (xrow[t] && at < k) xf[u][t] = *reinterpret_cast<const tp_bf16x8*>(xrow[t] + at);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int a = 0; a < ACCS; ++a) acc[t][a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][a], xf[u][t], acc[t][a], 0, 0, 0);
+  }
+}

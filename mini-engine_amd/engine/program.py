@@ -324,7 +324,7 @@ class StepProgram:
         dtype; ``sink`` float32 ``[heads]`` or None; pages of one key/value head with keys of ``rank + rotary_dim`` and values
         of ``rank`` elements. Returns the value ``[tokens, heads * value_dim]``, gated."""
         cols = heads * (head_dim + rotary_dim) + rank + rotary_dim + heads
-        if self._value_kinds[proj] != (cols, self.elem):
+        if self._value_kinds[proj][0] < cols or self._value_kinds[proj][1] != self.elem:  # (columns of padding may follow)
             raise ValueError(f"the projections have {self._value_kinds[proj][0]} columns, not {cols}")
         self._want(latent_norm, torch.float32, (rank,), "weight of the latent's norm")
         self._want(rope, torch.float32, None, "rotary table")

@@ -66,7 +66,11 @@ class LatentAttention(Mixer):
     def load(self, tensors, prefix: str) -> None:
         s, n = self.spec, self._n
         q = tensors[f"{prefix}.{n['q']}"]
-        self.w_in = torch.cat((q, tensors[f"{prefix}.{n['dkv']}"], tensors[f"{prefix}.{n['g']}"]), dim=0)
+        rows = [q, tensors[f"{prefix}.{n['dkv']}"], tensors[f"{prefix}.{n['g']}"]]
+        pad = -sum(t.shape[0] for t in rows) % 8  # rows of zeros: every token's projections then start at a multiple of 16 bytes
+        if pad:
+            rows.append(torch.zeros((pad, q.shape[1]), dtype=q.dtype, device=q.device))
+        self.w_in = torch.cat(rows, dim=0)
         self.w_o = tensors[f"{prefix}.{n['o']}"]
         # the keys' map per head, transposed: [heads, rank, d] reads a head's query part and gives its image in the latent space
         self.key_map = tensors[f"{prefix}.{n['uk']}"].view(self.nh, self.d, self.rank).transpose(1, 2).contiguous()
