@@ -180,6 +180,72 @@ __global__ __launch_bounds__(256) void routed_tile_mfma_kernel(const bf16_t* __r
   }
 }
 
+// Tiles of up to 16 pairs (decode steps): a block takes 16 columns of a tile and its four waves cut k among them in
+// interleaved chunks of 32 (a wave alone walks a row of weights in k / 64 dependent trips to memory; four waves in a
+// quarter of them), then add their sums up through LDS in the order of the waves. Otherwise as the kernel above.
+template <bool GATED>
+__global__ __launch_bounds__(256) void routed_tile_ksplit_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
+                                                                 const int* __restrict__ plan, const int* __restrict__ sorted,
+                                                                 const float* __restrict__ wts, bf16_t* __restrict__ acts,
+                                                                 float* __restrict__ parts, int num_tokens, int N, int K, int top,
+                                                                 int act) {
+  constexpr int ACCS = GATED ? 2 : 1, WAVES = 4, U = 2;
+  __shared__ float red[WAVES][ACCS][64][4];
+  const int tile = blockIdx.x;
+  if (tile >= plan[0]) return;
+  const int e = plan[1 + 3 * tile], begin = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
+  const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1), r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.y * 16;
+  const bf16_t* w0 = n0 + r < N ? W + ((size_t)e * ACCS * N + n0 + r) * K : nullptr;
+  const bf16_t* w1 = GATED && w0 ? w0 + (size_t)N * K : nullptr;
+  const int pair = r < rows ? sorted[begin + r] : -1;
+  const bf16_t* xr = r < rows ? x + (GATED ? (size_t)(pair / top) : (size_t)(begin + r)) * K : nullptr;
+  tp_float4 acc[ACCS];
+#pragma unroll
+  for (int a = 0; a < ACCS; ++a) acc[a] = (tp_float4){0.f, 0.f, 0.f, 0.f};
+  const int chunks = (K + 31) / 32;
+  for (int c0 = wave; c0 < chunks; c0 += WAVES * U) {
+    tp_bf16x8 wf[U][ACCS], xf[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + WAVES * u, at = c * 32 + 8 * g;
+      const bool k_ok = c < chunks && at < K;
+      wf[u][0] = tp_bf16x8{};
+      if (w0 && k_ok) wf[u][0] = *reinterpret_cast<const tp_bf16x8*>(w0 + at);
+      if (GATED) {
+        wf[u][ACCS - 1] = tp_bf16x8{};
+        if (w1 && k_ok) wf[u][ACCS - 1] = *reinterpret_cast<const tp_bf16x8*>(w1 + at);
+      }
+      xf[u] = tp_bf16x8{};
+      if (xr && k_ok) xf[u] = *reinterpret_cast<const tp_bf16x8*>(xr + at);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int a = 0; a < ACCS; ++a) acc[a] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][a], xf[u], acc[a], 0, 0, 0);
+  }
+#pragma unroll
+  for (int a = 0; a < ACCS; ++a)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) red[wave][a][lane][i] = acc[a][i];
+  __syncthreads();
+  if (wave != 0 || pair < 0) return;
+  float sum[ACCS][4];
+#pragma unroll
+  for (int a = 0; a < ACCS; ++a)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sum[a][i] = ((red[0][a][lane][i] + red[1][a][lane][i]) + red[2][a][lane][i]) + red[3][a][lane][i];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int col = n0 + 4 * g + i;
+    if (col >= N) continue;
+    if (GATED)
+      acts[(size_t)(begin + r) * N + col] = from_float<bf16_t>(gate_act(sum[0][i], act) * sum[ACCS - 1][i]);
+    else
+      parts[((size_t)(pair % top) * num_tokens + pair / top) * N + col] = wts[pair] * sum[0][i];
+  }
+}
+
 extern "C" int me_routed_ff_max_tiles(long long tokens, int E, int top) {
   return (int)((tokens * top + TP_ROWS - 1) / TP_ROWS) + E;
 }
@@ -221,6 +287,13 @@ extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, co
                                                                  nullptr, num_tokens, ff, hidden, top, act);
       routed_tile_mfma_kernel<4, false><<<g_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
                                                                   parts, num_tokens, hidden, ff, top, act);
+    } else if (P <= 4ll * E && (ff + 15) / 16 <= 65535 && (hidden + 15) / 16 <= 65535) {
+      // few pairs (decode steps): most tiles hold a pair or two, and what a step waits for is the walk over k
+      const dim3 k_up(max_tiles, (ff + 15) / 16), k_down(max_tiles, (hidden + 15) / 16);
+      routed_tile_ksplit_kernel<true><<<k_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
+                                                                nullptr, num_tokens, ff, hidden, top, act);
+      routed_tile_ksplit_kernel<false><<<k_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
+                                                                 parts, num_tokens, hidden, ff, top, act);
     } else {
       routed_tile_mfma_kernel<1, true><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
                                                                  nullptr, num_tokens, ff, hidden, top, act);

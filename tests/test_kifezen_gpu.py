@@ -248,11 +248,15 @@ def test_routed_experts_against_the_plain_mixture(hidden, ff, experts, top, toke
     assert got.parts.shape == (top, tokens, hidden)
     want = plain.routed_ff(h.to(F64), {"router": {"experts": experts, "top": top}}, {k: v.to(F64) for k, v in w.items()}, "m")
     assert rel_err(got.parts.sum(0), want) < TOL[dtype]
-    # a token's result does not depend on its company: alone, and among others in another order, the same bits
-    alone = K.routed_ff(h[-1:].cuda().contiguous(), router, gate_up, down, top)
-    assert torch.equal(alone.parts[:, 0], got.parts[:, -1])
+    # a token's result does not depend on its company: among others in another order the same bits; alone the same bits in
+    # float32, and in bfloat16 the same but for the order of the float32 sums over k (a step of few pairs cuts k among waves)
     flipped = K.routed_ff(h.flip(0).cuda().contiguous(), router, gate_up, down, top)
     assert torch.equal(flipped.parts.flip(1), got.parts)
+    alone = K.routed_ff(h[-1:].cuda().contiguous(), router, gate_up, down, top)
+    if dtype is torch.float32:
+        assert torch.equal(alone.parts[:, 0], got.parts[:, -1])
+    else:
+        assert rel_err(alone.parts[:, 0], got.parts[:, -1]) < 1e-5
 
 
 # --------------------------------------------------------------------------------- models through the engine
