@@ -398,6 +398,8 @@ def design_line(args) -> dict:
 
     design = args.design
     arch_name, config_of = DESIGNS[design]
+    batches = [int(b) for b in args.design_batches.split(",") if b]
+    headline = 8 if 8 in batches else batches[0]
     ctx, out = 2304, {}
     sizes = [z for z in args.design_sizes.split(",") if z]
     for size in sizes:
@@ -408,11 +410,11 @@ def design_line(args) -> dict:
         for name, arch, cfg in ((design, arch_name, config_of(size)), ("qwen3", "Qwen3ForCausalLM", qwen)):
             if args.design_alone and name == "qwen3":
                 continue
-            bench = DecodeBench(cfg, args.dtype, ctx, 64, architecture=arch)
+            bench = DecodeBench(cfg, args.dtype, ctx, max(batches), architecture=arch)
             pf = bench.prefill(args.prefill_tokens)
             out[f"{name}_{size}_prefill_{pf['tokens']}_tok_s"] = pf["value"]
             out[f"{name}_{size}_prefill_{pf['tokens']}_ms"] = pf["ms"]
-            for b in (1, 8, 64):
+            for b in batches:
                 m = bench.decode(b, args.steps, args.warmup)
                 out[f"{name}_{size}_decode_b{b}_tok_s"] = round(m[0], 1)
                 out[f"{name}_{size}_decode_b{b}_ms_per_step"] = round(m[1], 4)
@@ -420,13 +422,13 @@ def design_line(args) -> dict:
             del bench
             release()
     first = sizes[0]
-    return {"metric": f"decode tok/s at batch 8 ({arch_name} design, width {DESIGN_SIZES[first]['width']}, {DESIGN_LAYERS} layers)",
-            "value": out[f"{design}_{first}_decode_b8_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-            "warmup": args.warmup, "ms_per_step": out[f"{design}_{first}_decode_b8_ms_per_step"], "higher_is_better": True,
+    return {"metric": f"decode tok/s at batch {headline} ({arch_name} design, width {DESIGN_SIZES[first]['width']}, {DESIGN_LAYERS} layers)",
+            "value": out[f"{design}_{first}_decode_b{headline}_tok_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": out[f"{design}_{first}_decode_b{headline}_ms_per_step"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
             "data": "synthetic: seeded uniform-random token ids, random N(0, 0.02) weights",
             "config": {"model": f"{arch_name} design beside the Qwen3 dense design at equal layer sizes", "layers": DESIGN_LAYERS,
-                       "vocab": DESIGN_VOCAB, "sizes": {z: DESIGN_SIZES[z] for z in sizes}, "seq_len": ctx, "global_batch": 8,
+                       "vocab": DESIGN_VOCAB, "sizes": {z: DESIGN_SIZES[z] for z in sizes}, "seq_len": ctx, "global_batch": headline,
                        "parallelism": "single GPU"},
             "points": out}
 
@@ -448,6 +450,7 @@ def main() -> int:
     ap.add_argument("--design", default="", choices=["", "gonurax", "kifezen"],
                     help="instead of the default workload: this design beside the Qwen3 dense design at equal layer sizes")
     ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design to measure, comma separated")
+    ap.add_argument("--design-batches", default="1,8,64", help="decode batch sizes of --design, comma separated")
     ap.add_argument("--design-alone", action="store_true", help="profiling aid: --design without the Qwen3 model beside it")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -133,10 +133,15 @@ __global__ __launch_bounds__(256) void head_product_mfma_kernel(const bf16_t* __
     const int tok = t0 + t * 16 + r;
     if (tok >= num_tokens) continue;
     const float gv = gate ? 1.f / (1.f + expf(-to_float(gate[(size_t)tok * gate_row + h]))) : 1.f;
+    bf16_t* dst = out + (size_t)tok * out_row + (size_t)h * out_head + n0 + 4 * g;
+    if (n0 + 4 * g + 3 < n && (((uintptr_t)dst) & 7) == 0) {  // the lane's four columns as one store
+      typedef __bf16 hp_bf16x4 __attribute__((ext_vector_type(4)));
+      const hp_bf16x4 v = {(__bf16)(acc[t][0][0] * gv), (__bf16)(acc[t][0][1] * gv), (__bf16)(acc[t][0][2] * gv), (__bf16)(acc[t][0][3] * gv)};
+      *reinterpret_cast<hp_bf16x4*>(dst) = v;
+    } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int col = n0 + 4 * g + i;
-      if (col < n) out[(size_t)tok * out_row + (size_t)h * out_head + col] = from_float<bf16_t>(acc[t][0][i] * gv);
+      for (int i = 0; i < 4; ++i)
+        if (n0 + 4 * g + i < n) dst[i] = from_float<bf16_t>(acc[t][0][i] * gv);
     }
   }
 }

@@ -11,20 +11,33 @@
 // what else the step holds. Everything stays on the device: a step that a graph replays routes anew every time.
 #include "tile_product.h"
 
+extern "C" int me_gemm_grouped_tile_rows();
+extern "C" int me_gemm_grouped_bf16(const void* X, const void* W, const int* plan, const int* sorted, const float* wts, void* acts,
+                                    float* parts, int num_tokens, int N, int K, int top, int max_tiles, int gated, hipStream_t stream);
+
 #define RF_MAX_EXPERTS 1024
 #define RF_MAX_TOP 32
 
 template <typename T>
-__global__ __launch_bounds__(256) void routed_route_kernel(const T* __restrict__ h, const float* __restrict__ Wr, int* __restrict__ ids,
+__global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict__ h, const float* __restrict__ Wr, int* __restrict__ ids,
                                                            float* __restrict__ wts, int hidden, int E, int top) {
   __shared__ float z[RF_MAX_EXPERTS];
   const int t = blockIdx.x, wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const T* row = h + (size_t)t * hidden;
-  for (int e = wave; e < E; e += 4) {
+  // a wave an expert at a time; a lane's elements lie 64 apart, four of them in flight together with sums of their own
+  const int waves = blockDim.x / ME_WAVE;
+  for (int e = wave; e < E; e += waves) {
     const float* w = Wr + (size_t)e * hidden;
-    float s = 0.f;
-    for (int c = lane; c < hidden; c += ME_WAVE) s = fmaf(to_float(row[c]), w[c], s);
-    s = wave_sum(s);
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int c = lane;
+    for (; c + 3 * ME_WAVE < hidden; c += 4 * ME_WAVE) {
+      const float x0 = to_float(row[c]), x1 = to_float(row[c + ME_WAVE]), x2 = to_float(row[c + 2 * ME_WAVE]),
+                  x3 = to_float(row[c + 3 * ME_WAVE]);
+      const float w0 = w[c], w1 = w[c + ME_WAVE], w2 = w[c + 2 * ME_WAVE], w3 = w[c + 3 * ME_WAVE];
+      s0 = fmaf(x0, w0, s0), s1 = fmaf(x1, w1, s1), s2 = fmaf(x2, w2, s2), s3 = fmaf(x3, w3, s3);
+    }
+    for (; c < hidden; c += ME_WAVE) s0 = fmaf(to_float(row[c]), w[c], s0);
+    const float s = wave_sum((s0 + s1) + (s2 + s3));
     if (lane == 0) z[e] = s;
   }
   __syncthreads();
@@ -275,10 +288,19 @@ extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, co
   const dim3 g_up(max_tiles, (ff + TP_COLS - 1) / TP_COLS), g_down(max_tiles, (hidden + TP_COLS - 1) / TP_COLS);
   if (g_up.y > 65535 || g_down.y > 65535) return me_fail("me_routed_ff: hidden=%d ff=%d", hidden, ff);
   (void)elem;
+  // few tokens (decode steps): a wave an expert, so that all of a token's logits are on their way at once
+  const int route_threads = num_tokens <= 64 ? 64 * (E < 16 ? (E < 4 ? 4 : E) : 16) : 256;
   const bool aligned = ((((uintptr_t)h | (uintptr_t)W_gu | (uintptr_t)W_down | (uintptr_t)acts) & 15) == 0);
   if (dtype == ME_BF16 && hidden % 8 == 0 && ff % 8 == 0 && aligned) {  // the matrix cores
     const int wide = P >= 32ll * E;  // 32 and more pairs an expert on average: tiles of 64 pairs
-    routed_route_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
+    routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
+    if (P >= 96ll * E && hidden % 64 == 0 && ff % 64 == 0) {
+      // prompts: tiles of 128 pairs through the product that stages both operands in LDS (gemm_grouped.hip)
+      const int rows128 = me_gemm_grouped_tile_rows(), tiles128 = (int)((P + rows128 - 1) / rows128) + E;
+      routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, rows128, plan, sorted);
+      if (me_gemm_grouped_bf16(h, W_gu, plan, sorted, wts, acts, nullptr, num_tokens, ff, hidden, top, tiles128, act, stream)) return 1;
+      return me_gemm_grouped_bf16(acts, W_down, plan, sorted, wts, nullptr, parts, num_tokens, hidden, ff, top, tiles128, 0, stream);
+    }
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, wide ? 64 : 16, plan, sorted);
     if (wide) {
       const unsigned tiles64 = (unsigned)((P + 63) / 64) + E;  // fewer tiles than the list's bound: whole blocks that only return
@@ -303,14 +325,14 @@ extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, co
     return me_check_launch("me_routed_ff");
   }
   if (dtype == ME_F32) {
-    routed_route_kernel<float><<<num_tokens, 256, 0, stream>>>((const float*)h, Wr, ids, wts, hidden, E, top);
+    routed_route_kernel<float><<<num_tokens, route_threads, 0, stream>>>((const float*)h, Wr, ids, wts, hidden, E, top);
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, TP_ROWS, plan, sorted);
     routed_gate_up_kernel<float><<<g_up, 256, 0, stream>>>((const float*)h, (const float*)W_gu, plan, sorted, (float*)acts, hidden, ff,
                                                             top, act);
     routed_down_kernel<float><<<g_down, 256, 0, stream>>>((const float*)acts, (const float*)W_down, plan, sorted, wts, parts,
                                                           num_tokens, hidden, ff, top);
   } else {
-    routed_route_kernel<bf16_t><<<num_tokens, 256, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
+    routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, TP_ROWS, plan, sorted);
     routed_gate_up_kernel<bf16_t><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, (bf16_t*)acts, hidden,
                                                              ff, top, act);

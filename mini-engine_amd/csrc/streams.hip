@@ -55,6 +55,7 @@ __global__ void streams_norm_kernel(float* __restrict__ xs, size_t per_stream, i
   const size_t base = (size_t)src * dim;
   float ss = 0.f;
   for (int c = threadIdx.x; c < dim; c += blockDim.x) {
+    // every load of the element is asked for before the first is used: the streams, the result, its partial sums eight at a time
     float old[ME_MAX_STREAMS];
 #pragma unroll
     for (int s = 0; s < ME_MAX_STREAMS; ++s) old[s] = s < S ? xs[(size_t)s * per_stream + base + c] : 0.f;
@@ -62,8 +63,15 @@ __global__ void streams_norm_kernel(float* __restrict__ xs, size_t per_stream, i
     if (mix_out) {
       float y = delta ? to_float(delta[base + c]) : 0.f;
       if (parts) {
-        float d = parts[base + c];
-        for (int p = 1; p < num_parts; ++p) d += parts[(size_t)p * part_stride + base + c];
+        float d = 0.f;
+        for (int p0 = 0; p0 < num_parts; p0 += 8) {
+          float v[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) v[q] = p0 + q < num_parts ? parts[(size_t)(p0 + q) * part_stride + base + c] : 0.f;
+#pragma unroll
+          for (int q = 0; q < 8; ++q)
+            if (p0 + q < num_parts) d = p0 + q == 0 ? v[q] : d + v[q];
+        }
         y += d;
       }
       for (int t = 0; t < S; ++t) {
@@ -98,7 +106,9 @@ extern "C" int me_streams_norm(float* xs, long long per_stream, int S, const voi
   if (dim <= 0 || dim > 16384) return me_fail("me_streams_norm: rows of %d elements, at most 16384", dim);
   if ((delta || parts) && !mix_out) return me_fail("me_streams_norm: a pending result needs its coefficients");
   if (parts && (num_parts < 1 || part_stride < (long long)dim)) return me_fail("me_streams_norm: %d partial sums", num_parts);
-  const int threads = dim >= 2048 ? 512 : (dim >= 512 ? 256 : (dim >= 128 ? 128 : 64));
+  // a thread an element up to 1,024 of them (all loads of a row in flight at once), then two, four, ..
+  // (many rows hide each other's loads: blocks of 256 then)
+  const int threads = num_rows >= 256 ? (dim >= 256 ? 256 : (dim + 63) / 64 * 64) : (dim >= 1024 ? 1024 : (dim + 63) / 64 * 64);
   const size_t lds = (size_t)dim * sizeof(float);
   if (lds > 48 * 1024) {
     const void* fn = dtype == ME_F32 ? (const void*)streams_norm_kernel<float> : (const void*)streams_norm_kernel<bf16_t>;

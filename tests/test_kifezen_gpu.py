@@ -231,7 +231,10 @@ def test_latent_attention_kernels_against_the_expanded_form(nh, d, r, dv, rank, 
 # ----------------------------------------------------------------------------------- routed experts
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("hidden,ff,experts,top,tokens", [(96, 40, 5, 2, 37), (64, 24, 16, 4, 150), (128, 48, 8, 1, 3), (80, 56, 3, 3, 1),
-                                                          (100, 20, 40, 6, 64)])
+                                                          (100, 20, 40, 6, 64),
+                                                          # bfloat16: tiles of 64 pairs; tiles of 128 through LDS (and one that is no
+                                                          # multiple of 64 wide, which stays with the smaller tiles)
+                                                          (128, 64, 4, 2, 100), (128, 192, 4, 2, 300), (192, 64, 3, 1, 700), (136, 72, 2, 2, 260)])
 def test_routed_experts_against_the_plain_mixture(hidden, ff, experts, top, tokens, dtype):
     from mini_engine_amd.ops import kernels as K
 
