@@ -79,8 +79,10 @@ const CachedPlan& plan_for(Runner& r, const std::vector<int>& geometry) {
   CachedPlan fresh;
   fresh.key = key;
   const int items = (int)r.starts.size(), group = nh / nkv;
-  const bool wide = me::wide_blocks_pay(r.starts.data(), r.qlens.data(), items,
-                                        std::max(1, me_attention_prefill_columns(1) / group), window, nkv, r.compute_units);
+  // (heads of 256: the wide block's accumulators, 32 columns a wave, no longer fit the vector registers; see the measurement
+  // beside the latent attention layers in the design notes)
+  const bool wide = d < 256 && me::wide_blocks_pay(r.starts.data(), r.qlens.data(), items,
+                                                   std::max(1, me_attention_prefill_columns(1) / group), window, nkv, r.compute_units);
   fresh.columns = me_attention_prefill_columns(wide ? 1 : 0);
   me::build_work_list(r.starts.data(), r.qlens.data(), items, fresh.columns / group, window, nkv, r.compute_units,
                       (long long)nh * d * 4, fresh.list, keep_first);
