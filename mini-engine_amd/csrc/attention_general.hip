@@ -21,7 +21,8 @@
 // [positions, 2, dv/2]): the output of a token at position p, a sum of such values, is turned back by p's angles.
 #include "common.h"
 
-#define AG_MAX_D 256
+#define AG_MAX_D 256   // the kernels' usual instance: heads of up to 256 elements
+#define AG_MAX_D_WIDE 512  // a second instance of the kernel with a wave per token and head: up to 512
 
 #define AG_CHUNK 256  // keys per chunk
 
@@ -40,16 +41,16 @@ __device__ __forceinline__ void ag_merge(float& mt, float& lt, float (&acct)[KMA
 
 // `wpu` waves per (token, head): 1 (a block of four waves serves four of them), or all waves of the block for one,
 // which then take the chunks in turns, a round of wpu chunks at a time, and wave 0 merges the round's results in order.
-template <typename T>
+template <typename T, int KMAX>
 __global__ __launch_bounds__(512) void attention_general_kernel(
     const T* __restrict__ q, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ token_item, const int* __restrict__ block_table,
     int table_width, T* __restrict__ out, int num_tokens, int nh, int nkv, int d, int dv, int bs, int window, int keep_first,
     const float* __restrict__ unturn, int un_pairing, float scale, int wpu, const float* __restrict__ sink,
     const T* __restrict__ gate, size_t gate_row) {
-  constexpr int KMAX = AG_MAX_D / ME_WAVE;
-  __shared__ float qs[8][AG_MAX_D];
-  __shared__ float parts[8][AG_MAX_D + 2];  // with several waves per unit: a round's results (values, maximum, sum)
+  constexpr int DMAX = KMAX * ME_WAVE;  // the largest head this instance takes
+  __shared__ float qs[8][DMAX];
+  __shared__ float parts[8][DMAX + 2];  // with several waves per unit: a round's results (values, maximum, sum)
   const int wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const int w = wave % wpu;
   const long long unit = (long long)blockIdx.x * (blockDim.x / ME_WAVE / wpu) + wave / wpu;
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
       const float alpha = expf(m - m_new);  // exp(-inf) = 0 on the first tile
       l = l * alpha + wave_sum(pr);
 #pragma unroll
-      for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) acc[k] *= alpha;
+      for (int k = 0; k < KMAX; ++k) acc[k] *= alpha;
       m = m_new;
       const int j_lo = vlo > tile ? vlo - tile : 0;
       const int j_hi = vhi - tile < 63 ? vhi - tile : 63;
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
           const int kj = tile + j;
           const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
-          for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
+          for (int k = 0; k < KMAX; ++k) {
             const int i = lane + k * ME_WAVE;
             if (i < dv) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
           }
@@ -143,14 +144,14 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
         // eight groups of four keys at a time: their values are requested before the first is used
         const int groups = j <= j_hi ? (j_hi + 1 - j) / 4 : 0;  // whole groups from j on
         for (int g0 = 0; g0 < groups; g0 += 8) {
-          float4 vv[8][AG_MAX_D / ME_WAVE];
+          float4 vv[8][KMAX];
 #pragma unroll
           for (int gq = 0; gq < 8; ++gq) {
             const bool there = g0 + gq < groups;
             const int kj = tile + j + 4 * (there ? g0 + gq : 0);
             const T* vbase = v_cache + ((size_t)table[kj / bs] * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
-            for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
+            for (int k = 0; k < KMAX; ++k) {
               const int i = lane + k * ME_WAVE;
               vv[gq][k] = make_float4(0.f, 0.f, 0.f, 0.f);
               if (there && i < dv) vv[gq][k] = *reinterpret_cast<const float4*>(vbase + (size_t)i * bs);
@@ -163,7 +164,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
               const float p0 = __shfl(pr, jj, ME_WAVE), p1 = __shfl(pr, jj + 1, ME_WAVE), p2 = __shfl(pr, jj + 2, ME_WAVE),
                           p3 = __shfl(pr, jj + 3, ME_WAVE);
 #pragma unroll
-              for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
+              for (int k = 0; k < KMAX; ++k) {
                 if (lane + k * ME_WAVE < dv) {
                   acc[k] = fmaf(p0, vv[gq][k].x, acc[k]);
                   acc[k] = fmaf(p1, vv[gq][k].y, acc[k]);
@@ -182,7 +183,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
         const int page = table[kj / bs];
         const T* vbase = v_cache + ((size_t)page * nkv + kvh) * dv * bs + kj % bs;
 #pragma unroll
-        for (int k = 0; k < AG_MAX_D / ME_WAVE; ++k) {
+        for (int k = 0; k < KMAX; ++k) {
           const int i = lane + k * ME_WAVE;
           if (i < dv) acc[k] = fmaf(pj, to_float(vbase[(size_t)i * bs]), acc[k]);
         }
@@ -194,7 +195,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
       if (ci < n_chunks) {
 #pragma unroll
         for (int k = 0; k < KMAX; ++k) parts[w][lane + k * ME_WAVE] = acc[k];
-        if (lane == 0) parts[w][AG_MAX_D] = m, parts[w][AG_MAX_D + 1] = l;
+        if (lane == 0) parts[w][DMAX] = m, parts[w][DMAX + 1] = l;
       }
       __syncthreads();
       if (w == 0)
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(512) void attention_general_kernel(
           float accc[KMAX];
 #pragma unroll
           for (int k = 0; k < KMAX; ++k) accc[k] = parts[o][lane + k * ME_WAVE];
-          ag_merge<KMAX>(mt, lt, acct, parts[o][AG_MAX_D], parts[o][AG_MAX_D + 1], accc);
+          ag_merge<KMAX>(mt, lt, acct, parts[o][DMAX], parts[o][DMAX + 1], accc);
         }
       __syncthreads();
     }
@@ -464,12 +465,13 @@ extern "C" int me_attention_general_gated(const void* q, const void* k_cache, co
                                           const float* unturn, int un_pairing, float scale, const float* sink, const void* gate,
                                           long long gate_row, int dtype, int items, hipStream_t stream) {
   if (num_tokens <= 0) return 0;
-  if (d <= 0 || d > AG_MAX_D) return me_fail("me_attention_general: head_dim=%d must be in 1..%d", d, AG_MAX_D);
-  if (dv <= 0 || dv > AG_MAX_D) return me_fail("me_attention_general: value head size %d must be in 1..%d", dv, AG_MAX_D);
+  if (d <= 0 || d > AG_MAX_D_WIDE) return me_fail("me_attention_general: head_dim=%d must be in 1..%d", d, AG_MAX_D_WIDE);
+  if (dv <= 0 || dv > AG_MAX_D_WIDE) return me_fail("me_attention_general: value head size %d must be in 1..%d", dv, AG_MAX_D_WIDE);
+  const bool big = d > AG_MAX_D || dv > AG_MAX_D;  // the instance with eight elements a lane
   if (keep_first < 0 || (keep_first > 0 && window <= 0))
     return me_fail("me_attention_general: keep_first=%d needs a window", keep_first);
   if (unturn && (dv % 2 || (un_pairing & ~1))) return me_fail("me_attention_general: values of size %d, pairing %d", dv, un_pairing);
-  const bool plain = dv == d && keep_first == 0 && !unturn && !sink && !gate;
+  const bool plain = dv == d && keep_first == 0 && !unturn && !sink && !gate && !big;
   if (nh <= 0 || nkv <= 0 || nh % nkv)
     return me_fail("me_attention_general: %d query heads are not a multiple of %d key/value heads", nh, nkv);
   if (bs <= 0 || table_width <= 0 || window < 0)
@@ -511,16 +513,22 @@ extern "C" int me_attention_general_gated(const void* q, const void* k_cache, co
   // few units (decode steps): a block of eight waves each, which share a token's chunks of keys; else four units a block
   const int wpu = units < 2048 ? 8 : 1, waves = units < 2048 ? 8 : 4;
   const unsigned blocks = (unsigned)((units + waves / wpu - 1) / (waves / wpu));
-  if (dtype == ME_F32)
-    attention_general_kernel<float><<<blocks, waves * 64, 0, stream>>>(
-        (const float*)q, (const float*)k_cache, (const float*)v_cache, positions, token_item, block_table,
-        table_width, (float*)out, num_tokens, nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu, sink,
-        (const float*)gate, (size_t)gate_row);
-  else
-    attention_general_kernel<bf16_t><<<blocks, waves * 64, 0, stream>>>(
-        (const bf16_t*)q, (const bf16_t*)k_cache, (const bf16_t*)v_cache, positions, token_item, block_table,
-        table_width, (bf16_t*)out, num_tokens, nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu, sink,
-        (const bf16_t*)gate, (size_t)gate_row);
+#define ME_AG_LAUNCH(TT, KK)                                                                                                   \
+  attention_general_kernel<TT, KK><<<blocks, waves * 64, 0, stream>>>(                                                         \
+      (const TT*)q, (const TT*)k_cache, (const TT*)v_cache, positions, token_item, block_table, table_width, (TT*)out, num_tokens, \
+      nh, nkv, d, dv, bs, window, keep_first, unturn, un_pairing, scale, wpu, sink, (const TT*)gate, (size_t)gate_row)
+  if (dtype == ME_F32) {
+    if (big)
+      ME_AG_LAUNCH(float, AG_MAX_D_WIDE / ME_WAVE);
+    else
+      ME_AG_LAUNCH(float, AG_MAX_D / ME_WAVE);
+  } else {
+    if (big)
+      ME_AG_LAUNCH(bf16_t, AG_MAX_D_WIDE / ME_WAVE);
+    else
+      ME_AG_LAUNCH(bf16_t, AG_MAX_D / ME_WAVE);
+  }
+#undef ME_AG_LAUNCH
   return me_check_launch("me_attention_general");
 }
 

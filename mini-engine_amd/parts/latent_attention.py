@@ -20,7 +20,7 @@ import torch
 from ..weights.loader import TensorWant
 from .base import MIXERS, POSITION_ENCODINGS, KVBinding, KVCacheNeed, Mixer
 
-MAX_KEY_DIM = 256  # what the attention kernel that takes every size allows for rank + rotary_dim
+MAX_KEY_DIM = 512  # what the attention kernel that takes every size allows for rank + rotary_dim
 MATRIX_CORE_KEY_DIMS = (32, 64, 96, 128, 192, 256)  # csrc/attention_mfma.hip: me_attention_mfma_supported
 
 

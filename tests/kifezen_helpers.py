@@ -69,10 +69,14 @@ def configs() -> dict[str, dict]:
         "E": model(260, 128, 2, 1e-6, [
             attention(8, 2, 64, 64, 0.125, q_temp=(0.3, 40), mlp=dense(160)),
             latent(16, 24, 32, 16, 96, 0.13, 1e4, scaling=(4.0, 128, 16.0, 1.0), mlp=moe(6, 2, 64))]),
+        # a latent wider than the model, whose cached key has more than 256 elements
+        "F": model(150, 64, 2, 1e-6, [
+            latent(2, 16, 16, 24, 272, 0.1, 1e4, mlp=dense(96)),
+            attention(2, 2, 32, 32, 0.18, mlp=moe(4, 2, 32))]),
     }
 
 
-BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16}
+BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16, "F": 16}
 
 
 def wants_of(cfg: dict):

@@ -161,7 +161,9 @@ def test_a_large_sink_silences_a_head_and_a_low_one_is_not_there(dtype):
 # -------------------------------------------------------------------------------- latent attention
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("nh,d,r,dv,rank,bs,scaling", [(4, 32, 32, 32, 64, 16, (8.0, 2048, 32.0, 1.0)), (3, 16, 8, 24, 40, 8, (4.0, 64, 16.0, 2.0)),
-                                                        (5, 10, 6, 14, 18, 16, None), (2, 40, 16, 8, 200, 32, (2.0, 100, 8.0, 0.5))])
+                                                        (5, 10, 6, 14, 18, 16, None), (2, 40, 16, 8, 200, 32, (2.0, 100, 8.0, 0.5)),
+                                                        # a key of more than 256 elements: the attention kernel's wider instance
+                                                        (2, 24, 20, 16, 300, 16, None)])
 def test_latent_attention_kernels_against_the_expanded_form(nh, d, r, dv, rank, bs, scaling, dtype):
     """The projections of two sequences through the latent's norm, the rotation, the page write, the folded keys' map,
     attention with a sink and the values' map with the gate, whole and in portions, against the plain implementation
@@ -291,7 +293,7 @@ def requests_for(cfg, seed, lengths=(1, 23, 97, 150, 61)):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F"])
 def test_every_way_of_cutting_gives_the_plain_logits(folders, name, dtype):
     """Whole prompts; most of a prompt and its tail token by token (replayed graphs); portions down to two tokens; up
     to four live requests in a pool whose pages are used again: all against the plain implementation."""
