@@ -53,7 +53,7 @@ def configs() -> dict[str, dict]:
             latent(3, 16, 8, 24, 40, 0.17, 1e4, scaling=(4.0, 64, 16.0, 2.0), mlp=dense(136)),
             latent(2, 40, 16, 8, 24, 0.11, 500.0, mlp=moe(3, 3, 56))]),
         "B": model(500, 128, 1, 1e-6, [
-            latent(4, 32, 32, 32, 64, 0.125, 5e4, scaling=(8.0, 256, 32.0, 1.0), mlp=moe(8, 1, 48)),
+            latent(4, 24, 40, 32, 56, 0.15, 3e4, scaling=(6.0, 256, 24.0, 1.0), mlp=moe(8, 1, 48)),
             attention(6, 6, 20, 20, 0.22, q_temp=(0.25, 100)),
             attention(2, 1, 64, 40, 0.09, mlp=dense(192))]),
         "C": model(131, 80, 4, 1e-6, [

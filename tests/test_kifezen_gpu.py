@@ -76,7 +76,7 @@ def shuffled_table(items_len: list[int], bs: int, seed: int):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("nh,nkv,d,dv,bs", [(4, 2, 48, 48, 16), (6, 1, 20, 36, 8), (3, 3, 64, 16, 32)])
+@pytest.mark.parametrize("nh,nkv,d,dv,bs", [(8, 2, 40, 40, 16), (6, 1, 20, 36, 8), (3, 3, 64, 16, 32)])
 def test_unit_norm_temperature_gate_and_sink_in_attention(nh, nkv, d, dv, bs, dtype):
     """Two sequences in one step, a prompt and a prompt's portion behind cached keys: q and k over their root mean square,
     the query's temperature at the positions where it steps, the gate, a sink; one key far back that outweighs hundreds."""
@@ -160,7 +160,7 @@ def test_a_large_sink_silences_a_head_and_a_low_one_is_not_there(dtype):
 
 # -------------------------------------------------------------------------------- latent attention
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("nh,d,r,dv,rank,bs,scaling", [(4, 32, 32, 32, 64, 16, (8.0, 2048, 32.0, 1.0)), (3, 16, 8, 24, 40, 8, (4.0, 64, 16.0, 2.0)),
+@pytest.mark.parametrize("nh,d,r,dv,rank,bs,scaling", [(4, 24, 16, 40, 48, 16, (6.0, 1024, 24.0, 2.0)), (3, 16, 8, 24, 40, 8, (4.0, 64, 16.0, 2.0)),
                                                         (5, 10, 6, 14, 18, 16, None), (2, 40, 16, 8, 200, 32, (2.0, 100, 8.0, 0.5)),
                                                         # a key of more than 256 elements: the attention kernel's wider instance
                                                         (2, 24, 20, 16, 300, 16, None)])
