@@ -756,7 +756,7 @@ static int decode_common(const void* q, const void* k_cache, const void* v_cache
   const int block_waves = decode_block_waves(items, nh, nkv, d, num_splits);
   if (!out && block_waves > 1)
     return me_fail("me_attention_decode_bf16: a launch whose blocks add up their splits themselves needs `out`");
-  if (!out && sink) return me_fail("me_attention_decode_bf16: the product that adds up the splits itself knows no sink");
+  // (without `out` the caller adds up the splits and owes them the sink: me_latent_values_bf16)
   const int cus = decode_compute_units();
   const long long blocks = (long long)items * nkv * ((nh / nkv + 15) / 16);
   // Keys and values pass through once: loaded as non-temporal they arrive faster where the launch streams hundreds of

@@ -692,9 +692,17 @@ class Run {
       const SplitPlan sp = split_plan(items, (nh + 15) / 16, s_.max_ctx, s_.least_live, idx(s_.lay.live_items));
       float* part_o = (float*)arena_.take((size_t)items * nh * sp.num_splits * dk * 4);
       float* part_ml = (float*)arena_.take((size_t)items * nh * sp.num_splits * 2 * 4);
-      ok(me_attention_decode_bf16_sink(qa, kc, vc, idx(s_.lay.item_ctx), table, width, ol, part_o, part_ml, items, nh, 1, dk, bs, sink,
-                                       scale, sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits, kDecodeWaves,
-                                       idx(s_.lay.live_items) + 1, stream_));
+      // where the launch leaves one partial result per split, one kernel adds them up (with the sink), maps the weighted
+      // latents to the heads' values and gates them: no kernel of its own for the sum, none for the values' map
+      const bool tail = me_attention_decode_leaves_parts(items, nh, 1, dk, sp.num_splits) && me_latent_values_supported(sp.num_splits, rank);
+      ok(me_attention_decode_bf16_sink(qa, kc, vc, idx(s_.lay.item_ctx), table, width, tail ? nullptr : ol, part_o, part_ml, items, nh, 1,
+                                       dk, bs, sink, scale, sp.split_keys, sp.num_splits, s_.max_ctx, sp.live, sp.full_splits,
+                                       kDecodeWaves, idx(s_.lay.live_items) + 1, stream_));
+      if (tail) {
+        ok(me_latent_values_bf16(part_o, part_ml, sp.num_splits, dk, rank, sink, op.p[5], proj + (size_t)(used - nh) * elem_, row,
+                                 bufs_[op.out], items, nh, dv, stream_));
+        return;
+      }
     } else if (latent_takes_matrix_cores(op, dtype_)) {
       auto it = s_.plans.find({nh, 1, dk, 0, 0});
       if (it == s_.plans.end()) throw Error(kBroken, "the step has no work list for a latent attention layer");

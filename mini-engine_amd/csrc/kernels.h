@@ -110,6 +110,9 @@ int me_latent_prepare(const void* proj, long long row_stride, const float* norm_
 int me_head_product(const void* x, long long x_row, long long x_head, const void* W, void* out, long long out_row,
                     long long out_head, const void* gate, long long gate_row, int num_tokens, int heads, int n, int k, int dtype,
                     hipStream_t stream);
+int me_latent_values_supported(int num_splits, int rank);
+int me_latent_values_bf16(const float* part_o, const float* part_ml, int num_splits, int dk, int rank, const float* sink, const void* W_uv,
+                          const void* gate, long long gate_row, void* out, int items, int nh, int dv, hipStream_t stream);
 int me_head_gate(void* rows, const void* gate, long long gate_row, int num_tokens, int heads, int n, int dtype, hipStream_t stream);
 int me_routed_ff_max_tiles(long long tokens, int E, int top);
 long long me_routed_ff_workspace(long long tokens, int E, int top, int ff, int elem);

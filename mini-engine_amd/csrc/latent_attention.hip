@@ -198,3 +198,91 @@ extern "C" int me_head_gate(void* rows, const void* gate, long long gate_row, in
     head_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)rows, (const bf16_t*)gate, (size_t)gate_row, heads, n, total);
   return me_check_launch("me_head_gate");
 }
+
+// A decode step's tail of a latent attention layer in one kernel: the sum over the splits of the split-context attention
+// kernel (their unnormalised weighted latents part_o [item, head, split, dk] and statistics part_ml [.., 2] = (maximum in
+// units of log2, sum), with the sink as one more split of weight 1 and no value), the result rounded to bfloat16 as the
+// kernel that adds up splits rounds it, then the head's values' map and its gate:
+//   out[item, head, :] = sigmoid(gate[item, head]) * W_uv[head] . round(sum_s w_s o_s[:rank] / sum_s w_s l_s)
+// One block of 256 threads per (item, head).
+#define LV_MAX_SPLITS 1024
+#define LV_MAX_RANK 512
+__global__ __launch_bounds__(256) void latent_values_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                            int num_splits, int dk, int rank, const float* __restrict__ sink,
+                                                            const bf16_t* __restrict__ W_uv, const bf16_t* __restrict__ gate,
+                                                            size_t gate_row, bf16_t* __restrict__ out, int nh, int dv) {
+  __shared__ float wgt[LV_MAX_SPLITS];
+  __shared__ float lat[LV_MAX_RANK];
+  __shared__ float red_max[4], red_sum[4];
+  const size_t unit = blockIdx.x;
+  const int item = (int)(unit / nh), head = (int)(unit % nh);
+  const int tid = threadIdx.x, lane = tid & (ME_WAVE - 1), wave = tid / ME_WAVE;
+  const float* ml = part_ml + unit * num_splits * 2;
+  float big = -INFINITY;
+  for (int s = tid; s < num_splits; s += 256)
+    if (ml[s * 2 + 1] > 0.f) big = fmaxf(big, ml[s * 2]);
+  big = wave_max(big);
+  if (lane == 0) red_max[wave] = big;
+  __syncthreads();
+  big = fmaxf(fmaxf(red_max[0], red_max[1]), fmaxf(red_max[2], red_max[3]));
+  const float s2 = sink ? sink[head] * 1.4426950408889634f : -INFINITY;
+  big = fmaxf(big, s2);
+  float part_denom = 0.f;
+  for (int s = tid; s < num_splits; s += 256) {
+    const float l = ml[s * 2 + 1];
+    const float w = l > 0.f ? exp2f(ml[s * 2] - big) : 0.f;  // an empty split has no weight
+    wgt[s] = w;
+    part_denom += w * l;
+  }
+  part_denom = wave_sum(part_denom);
+  if (lane == 0) red_sum[wave] = part_denom;
+  __syncthreads();
+  const float denom = (red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]) + (sink ? exp2f(s2 - big) : 0.f);
+  const float inv = denom > 0.f ? 1.f / denom : 0.f;
+  const float* po = part_o + unit * num_splits * dk;
+  for (int c = tid; c < rank; c += 256) {
+    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+    int s = 0;
+    for (; s + 3 < num_splits; s += 4) {  // four splits' loads in flight together
+      const float v0 = po[(size_t)s * dk + c], v1 = po[(size_t)(s + 1) * dk + c], v2 = po[(size_t)(s + 2) * dk + c],
+                  v3 = po[(size_t)(s + 3) * dk + c];
+      a0 = fmaf(wgt[s], v0, a0), a1 = fmaf(wgt[s + 1], v1, a1), a2 = fmaf(wgt[s + 2], v2, a2), a3 = fmaf(wgt[s + 3], v3, a3);
+    }
+    for (; s < num_splits; ++s) a0 = fmaf(wgt[s], po[(size_t)s * dk + c], a0);
+    lat[c] = to_float(from_float<bf16_t>(((a0 + a1) + (a2 + a3)) * inv));
+  }
+  __syncthreads();
+  const float gv = gate ? 1.f / (1.f + expf(-to_float(gate[(size_t)item * gate_row + head]))) : 1.f;
+  const bool wide = rank % 8 == 0 && (((uintptr_t)W_uv) & 15) == 0;
+  for (int j = tid; j < dv; j += 256) {
+    const bf16_t* w = W_uv + ((size_t)head * dv + j) * rank;
+    float acc = 0.f;
+    if (wide) {
+      for (int c = 0; c < rank; c += 8) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(w + c);
+        const unsigned u[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          acc = fmaf(__uint_as_float(u[q] << 16), lat[c + 2 * q], acc);
+          acc = fmaf(__uint_as_float(u[q] & 0xffff0000u), lat[c + 2 * q + 1], acc);
+        }
+      }
+    } else {
+      for (int c = 0; c < rank; ++c) acc = fmaf(to_float(w[c]), lat[c], acc);
+    }
+    out[unit * dv + j] = from_float<bf16_t>(acc * gv);
+  }
+}
+
+extern "C" int me_latent_values_supported(int num_splits, int rank) { return num_splits <= LV_MAX_SPLITS && rank <= LV_MAX_RANK; }
+
+extern "C" int me_latent_values_bf16(const float* part_o, const float* part_ml, int num_splits, int dk, int rank, const float* sink,
+                                     const void* W_uv, const void* gate, long long gate_row, void* out, int items, int nh, int dv,
+                                     hipStream_t stream) {
+  if (items <= 0) return 0;
+  if (!me_latent_values_supported(num_splits, rank) || num_splits < 1 || rank > dk || nh <= 0 || dv <= 0)
+    return me_fail("me_latent_values: splits=%d rank=%d dk=%d heads=%d dv=%d", num_splits, rank, dk, nh, dv);
+  latent_values_kernel<<<(unsigned)(items * nh), 256, 0, stream>>>(part_o, part_ml, num_splits, dk, rank, sink, (const bf16_t*)W_uv,
+                                                                   (const bf16_t*)gate, (size_t)gate_row, (bf16_t*)out, nh, dv);
+  return me_check_launch("me_latent_values");
+}

@@ -17,10 +17,12 @@ extern "C" int me_gemm_grouped_bf16(const void* X, const void* W, const int* pla
 
 #define RF_MAX_EXPERTS 1024
 #define RF_MAX_TOP 32
+#define RF_DIRECT_PAIRS 16  // steps of up to this many pairs (token, pick) are not sorted: a pair is a tile
 
 template <typename T>
 __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict__ h, const float* __restrict__ Wr, int* __restrict__ ids,
-                                                           float* __restrict__ wts, int hidden, int E, int top) {
+                                                            float* __restrict__ wts, int hidden, int E, int top,
+                                                            int* __restrict__ plan, int* __restrict__ sorted, int num_pairs) {
   __shared__ float z[RF_MAX_EXPERTS];
   const int t = blockIdx.x, wave = threadIdx.x / ME_WAVE, lane = threadIdx.x & (ME_WAVE - 1);
   const T* row = h + (size_t)t * hidden;
@@ -43,6 +45,7 @@ __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict_
   __syncthreads();
   if (wave != 0) return;
   float mine = 0.f, zmax = 0.f, sum = 0.f;  // lane j keeps the weight of the j-th pick
+  int mine_e = 0;
   for (int j = 0; j < top; ++j) {
     float best = -INFINITY;
     int at = 0x7fffffff;
@@ -57,7 +60,7 @@ __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict_
     if (at >= E) at = 0;  // (a row of NaNs, as rows that pad a replayed step may be: any expert)
     if (j == 0) zmax = best;
     const float p = expf(best - zmax);
-    if (lane == j) mine = p;
+    if (lane == j) mine = p, mine_e = at;
     sum += p;
     if (lane == 0) {
       ids[(size_t)t * top + j] = at;
@@ -67,6 +70,16 @@ __global__ __launch_bounds__(1024) void routed_route_kernel(const T* __restrict_
     __builtin_amdgcn_s_waitcnt(0xc07f);
   }
   if (lane < top) wts[(size_t)t * top + lane] = mine / sum;
+  // A step of very few pairs needs no sorting: every pair is a tile of its own, in the order of the pairs (plan and
+  // sorted as routed_sort_kernel leaves them for tiles of one row).
+  if (plan && lane < top) {
+    const int pair = t * top + lane;
+    plan[1 + 3 * pair] = mine_e;
+    plan[2 + 3 * pair] = pair;
+    plan[3 + 3 * pair] = 1;
+    sorted[pair] = pair;
+    if (pair == 0) plan[0] = num_pairs;
+  }
 }
 
 // plan: [0] number of tiles; [1 + 3 i ..] tile i: expert, first position, pairs; sorted [P]: the pair at each position.
@@ -260,7 +273,7 @@ __global__ __launch_bounds__(256) void routed_tile_ksplit_kernel(const bf16_t* _
 }
 
 extern "C" int me_routed_ff_max_tiles(long long tokens, int E, int top) {
-  return (int)((tokens * top + TP_ROWS - 1) / TP_ROWS) + E;
+  return (int)((tokens * top + TP_ROWS - 1) / TP_ROWS) + E + RF_DIRECT_PAIRS;  // (or a tile a pair, for steps of very few pairs)
 }
 
 // Bytes of workspace: ids and weights of the pairs, the tile list, the sorted pairs, the activations.
@@ -293,7 +306,17 @@ extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, co
   const bool aligned = ((((uintptr_t)h | (uintptr_t)W_gu | (uintptr_t)W_down | (uintptr_t)acts) & 15) == 0);
   if (dtype == ME_BF16 && hidden % 8 == 0 && ff % 8 == 0 && aligned) {  // the matrix cores
     const int wide = P >= 32ll * E;  // 32 and more pairs an expert on average: tiles of 64 pairs
-    routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
+    const bool direct = P <= RF_DIRECT_PAIRS && (ff + 15) / 16 <= 65535 && (hidden + 15) / 16 <= 65535;
+    routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top,
+                                                                            direct ? plan : nullptr, direct ? sorted : nullptr, (int)P);
+    if (direct) {  // the router has written the list of tiles itself
+      const dim3 k_up((unsigned)P, (ff + 15) / 16), k_down((unsigned)P, (hidden + 15) / 16);
+      routed_tile_ksplit_kernel<true><<<k_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, wts, (bf16_t*)acts,
+                                                                nullptr, num_tokens, ff, hidden, top, act);
+      routed_tile_ksplit_kernel<false><<<k_down, 256, 0, stream>>>((const bf16_t*)acts, (const bf16_t*)W_down, plan, sorted, wts, nullptr,
+                                                                 parts, num_tokens, hidden, ff, top, act);
+      return me_check_launch("me_routed_ff");
+    }
     if (P >= 96ll * E && hidden % 64 == 0 && ff % 64 == 0) {
       // prompts: tiles of 128 pairs through the product that stages both operands in LDS (gemm_grouped.hip)
       const int rows128 = me_gemm_grouped_tile_rows(), tiles128 = (int)((P + rows128 - 1) / rows128) + E;
@@ -325,14 +348,14 @@ extern "C" int me_routed_ff(const void* h, const float* Wr, const void* W_gu, co
     return me_check_launch("me_routed_ff");
   }
   if (dtype == ME_F32) {
-    routed_route_kernel<float><<<num_tokens, route_threads, 0, stream>>>((const float*)h, Wr, ids, wts, hidden, E, top);
+    routed_route_kernel<float><<<num_tokens, route_threads, 0, stream>>>((const float*)h, Wr, ids, wts, hidden, E, top, nullptr, nullptr, 0);
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, TP_ROWS, plan, sorted);
     routed_gate_up_kernel<float><<<g_up, 256, 0, stream>>>((const float*)h, (const float*)W_gu, plan, sorted, (float*)acts, hidden, ff,
                                                             top, act);
     routed_down_kernel<float><<<g_down, 256, 0, stream>>>((const float*)acts, (const float*)W_down, plan, sorted, wts, parts,
                                                           num_tokens, hidden, ff, top);
   } else {
-    routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top);
+    routed_route_kernel<bf16_t><<<num_tokens, route_threads, 0, stream>>>((const bf16_t*)h, Wr, ids, wts, hidden, E, top, nullptr, nullptr, 0);
     routed_sort_kernel<<<1, 1024, 0, stream>>>(ids, (int)P, E, max_tiles, TP_ROWS, plan, sorted);
     routed_gate_up_kernel<bf16_t><<<g_up, 256, 0, stream>>>((const bf16_t*)h, (const bf16_t*)W_gu, plan, sorted, (bf16_t*)acts, hidden,
                                                              ff, top, act);
