@@ -73,10 +73,14 @@ def configs() -> dict[str, dict]:
         "F": model(150, 64, 2, 1e-6, [
             latent(2, 16, 16, 24, 272, 0.1, 1e4, mlp=dense(96)),
             attention(2, 2, 32, 32, 0.18, mlp=moe(4, 2, 32))]),
+        # a cached key of 256 elements (the matrix-core kernels' largest head) under three streams; a key of 64 under one head
+        "G": model(180, 64, 3, 1e-5, [
+            latent(4, 16, 64, 16, 192, 0.08, 1e4, scaling=(16.0, 64, 8.0, 1.0), mlp=moe(3, 2, 40)),
+            latent(1, 32, 16, 48, 48, 0.2, 2e3, mlp=dense(80))]),
     }
 
 
-BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16, "F": 16}
+BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16, "F": 16, "G": 16}
 
 
 def wants_of(cfg: dict):
