@@ -212,25 +212,57 @@ __global__ __launch_bounds__(256) void latent_values_kernel(const float* __restr
                                                             const bf16_t* __restrict__ W_uv, const bf16_t* __restrict__ gate,
                                                             size_t gate_row, bf16_t* __restrict__ out, int nh, int dv) {
   __shared__ float wgt[LV_MAX_SPLITS];
-  __shared__ float lat[LV_MAX_RANK];
+  __shared__ __attribute__((aligned(16))) float lat[LV_MAX_RANK];
+  __shared__ __attribute__((aligned(16))) bf16_t latb[LV_MAX_RANK];  // the same, as the matrix cores read it
+  __shared__ float4 partial[256];
   __shared__ float red_max[4], red_sum[4];
   const size_t unit = blockIdx.x;
   const int item = (int)(unit / nh), head = (int)(unit % nh);
   const int tid = threadIdx.x, lane = tid & (ME_WAVE - 1), wave = tid / ME_WAVE;
   const float* ml = part_ml + unit * num_splits * 2;
-  float big = -INFINITY;
-  for (int s = tid; s < num_splits; s += 256)
+  const float* po = part_o + unit * num_splits * dk;
+  // what nothing has to be waited for is asked for first: this thread's first weights of the values' map, and its first
+  // partial results (thread -> four elements of the latent, one of 256 / (rank / 4) groups of splits)
+  constexpr int EARLY = 8;
+  // Loads come back in the order they were asked for: first what the kernel needs first (this thread's split's statistics and
+  // the sink), then its partial results, then the weights and the gate, which wait for the kernel's end.
+  const float m_mine = tid < num_splits ? ml[tid * 2] : -INFINITY, l_mine = tid < num_splits ? ml[tid * 2 + 1] : 0.f;
+  const float sink_raw = sink ? sink[head] : 0.f;
+  const bool wide = rank % 8 == 0 && (((uintptr_t)W_uv) & 15) == 0;
+  // (the values' map on the matrix cores: wave w takes the tiles of 16 columns w, w + 4, ..; lane (r, g) feeds row n0 + r of the
+  // map, eight elements from 32 c + 8 g; the one token's latent is row 0 of the other operand)
+  const int rr = lane & 15, gg = lane >> 4;
+  const bf16_t* wrow = wave * 16 + rr < dv ? W_uv + ((size_t)head * dv + wave * 16 + rr) * rank : nullptr;
+  const bool quads_ok = rank % 4 == 0 && dk % 4 == 0 && rank / 4 <= 256;
+  const int quads = quads_ok ? rank / 4 : 1, groups = quads_ok ? 256 / quads : 1;
+  const int qd = tid % quads, grp = tid / quads;
+  float4 early[EARLY];
+#pragma unroll
+  for (int i = 0; i < EARLY; ++i) {
+    const int sp = grp + i * groups;
+    early[i] = quads_ok && grp < groups && sp < num_splits ? *reinterpret_cast<const float4*>(po + (size_t)sp * dk + qd * 4)
+                                                           : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  tp_bf16x8 wpre[EARLY];
+#pragma unroll
+  for (int i = 0; i < EARLY; ++i) {
+    wpre[i] = tp_bf16x8{};
+    if (wide && wrow && 32 * i + 8 * gg < rank) wpre[i] = *reinterpret_cast<const tp_bf16x8*>(wrow + 32 * i + 8 * gg);
+  }
+  const float gate_raw = gate ? to_float(gate[(size_t)item * gate_row + head]) : 0.f;
+  float big = l_mine > 0.f ? m_mine : -INFINITY;
+  for (int s = tid + 256; s < num_splits; s += 256)
     if (ml[s * 2 + 1] > 0.f) big = fmaxf(big, ml[s * 2]);
   big = wave_max(big);
   if (lane == 0) red_max[wave] = big;
   __syncthreads();
   big = fmaxf(fmaxf(red_max[0], red_max[1]), fmaxf(red_max[2], red_max[3]));
-  const float s2 = sink ? sink[head] * 1.4426950408889634f : -INFINITY;
+  const float s2 = sink ? sink_raw * 1.4426950408889634f : -INFINITY;
   big = fmaxf(big, s2);
   float part_denom = 0.f;
   for (int s = tid; s < num_splits; s += 256) {
-    const float l = ml[s * 2 + 1];
-    const float w = l > 0.f ? exp2f(ml[s * 2] - big) : 0.f;  // an empty split has no weight
+    const float l = s == tid ? l_mine : ml[s * 2 + 1];
+    const float w = l > 0.f ? exp2f((s == tid ? m_mine : ml[s * 2]) - big) : 0.f;  // an empty split has no weight
     wgt[s] = w;
     part_denom += w * l;
   }
@@ -239,38 +271,83 @@ __global__ __launch_bounds__(256) void latent_values_kernel(const float* __restr
   __syncthreads();
   const float denom = (red_sum[0] + red_sum[1]) + (red_sum[2] + red_sum[3]) + (sink ? exp2f(s2 - big) : 0.f);
   const float inv = denom > 0.f ? 1.f / denom : 0.f;
-  const float* po = part_o + unit * num_splits * dk;
-  for (int c = tid; c < rank; c += 256) {
-    float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
-    int s = 0;
-    for (; s + 3 < num_splits; s += 4) {  // four splits' loads in flight together
-      const float v0 = po[(size_t)s * dk + c], v1 = po[(size_t)(s + 1) * dk + c], v2 = po[(size_t)(s + 2) * dk + c],
-                  v3 = po[(size_t)(s + 3) * dk + c];
-      a0 = fmaf(wgt[s], v0, a0), a1 = fmaf(wgt[s + 1], v1, a1), a2 = fmaf(wgt[s + 2], v2, a2), a3 = fmaf(wgt[s + 3], v3, a3);
+  if (quads_ok) {
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (grp < groups) {
+#pragma unroll
+      for (int i = 0; i < EARLY; ++i) {
+        const int sp = grp + i * groups;
+        const float w = sp < num_splits ? wgt[sp] : 0.f;
+        a.x = fmaf(w, early[i].x, a.x), a.y = fmaf(w, early[i].y, a.y), a.z = fmaf(w, early[i].z, a.z), a.w = fmaf(w, early[i].w, a.w);
+      }
+      for (int sp = grp + EARLY * groups; sp < num_splits; sp += groups) {
+        const float w = wgt[sp];
+        const float4 v = *reinterpret_cast<const float4*>(po + (size_t)sp * dk + qd * 4);
+        a.x = fmaf(w, v.x, a.x), a.y = fmaf(w, v.y, a.y), a.z = fmaf(w, v.z, a.z), a.w = fmaf(w, v.w, a.w);
+      }
     }
-    for (; s < num_splits; ++s) a0 = fmaf(wgt[s], po[(size_t)s * dk + c], a0);
-    lat[c] = to_float(from_float<bf16_t>(((a0 + a1) + (a2 + a3)) * inv));
+    partial[tid] = a;
+    __syncthreads();
+    if (tid < quads) {
+      float4 total = partial[tid];
+      for (int gi = 1; gi < groups; ++gi) {
+        const float4 v = partial[gi * quads + tid];
+        total.x += v.x, total.y += v.y, total.z += v.z, total.w += v.w;
+      }
+      lat[4 * tid] = to_float(from_float<bf16_t>(total.x * inv));
+      lat[4 * tid + 1] = to_float(from_float<bf16_t>(total.y * inv));
+      lat[4 * tid + 2] = to_float(from_float<bf16_t>(total.z * inv));
+      lat[4 * tid + 3] = to_float(from_float<bf16_t>(total.w * inv));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) latb[4 * tid + i] = from_float<bf16_t>(lat[4 * tid + i]);
+    }
+  } else {
+    for (int c = tid; c < rank; c += 256) {
+      float a0 = 0.f;
+      for (int s = 0; s < num_splits; ++s) a0 = fmaf(wgt[s], po[(size_t)s * dk + c], a0);
+      latb[c] = from_float<bf16_t>(a0 * inv);
+      lat[c] = to_float(latb[c]);
+    }
   }
   __syncthreads();
-  const float gv = gate ? 1.f / (1.f + expf(-to_float(gate[(size_t)item * gate_row + head]))) : 1.f;
-  const bool wide = rank % 8 == 0 && (((uintptr_t)W_uv) & 15) == 0;
-  for (int j = tid; j < dv; j += 256) {
-    const bf16_t* w = W_uv + ((size_t)head * dv + j) * rank;
-    float acc = 0.f;
-    if (wide) {
-      for (int c = 0; c < rank; c += 8) {
-        const uint4 raw = *reinterpret_cast<const uint4*>(w + c);
-        const unsigned u[4] = {raw.x, raw.y, raw.z, raw.w};
+  const float gv = gate ? 1.f / (1.f + expf(-gate_raw)) : 1.f;
+  if (wide) {
+    for (int n0 = wave * 16; n0 < dv; n0 += 64) {
+      const bf16_t* w = n0 + rr < dv ? W_uv + ((size_t)head * dv + n0 + rr) * rank : nullptr;
+      tp_float4 acc = {0.f, 0.f, 0.f, 0.f};
+      int k0 = 0;
+      if (n0 == wave * 16) {  // the wave's first tile: its first weights were asked for at the kernel's head
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          acc = fmaf(__uint_as_float(u[q] << 16), lat[c + 2 * q], acc);
-          acc = fmaf(__uint_as_float(u[q] & 0xffff0000u), lat[c + 2 * q + 1], acc);
+        for (int i = 0; i < EARLY; ++i) {
+          const int at = 32 * i + 8 * gg;
+          if (32 * i < rank) {
+            tp_bf16x8 xf = tp_bf16x8{};
+            if (rr == 0 && at < rank) xf = *reinterpret_cast<const tp_bf16x8*>(latb + at);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wpre[i], xf, acc, 0, 0, 0);
+          }
         }
+        k0 = 32 * EARLY;
       }
-    } else {
-      for (int c = 0; c < rank; ++c) acc = fmaf(to_float(w[c]), lat[c], acc);
+      for (; k0 < rank; k0 += 32) {
+        const int at = k0 + 8 * gg;
+        tp_bf16x8 wf = tp_bf16x8{}, xf = tp_bf16x8{};
+        if (w && at < rank) wf = *reinterpret_cast<const tp_bf16x8*>(w + at);
+        if (rr == 0 && at < rank) xf = *reinterpret_cast<const tp_bf16x8*>(latb + at);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf, acc, 0, 0, 0);
+      }
+      if (rr == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n0 + 4 * gg + i < dv) out[unit * dv + n0 + 4 * gg + i] = from_float<bf16_t>(acc[i] * gv);
+      }
     }
-    out[unit * dv + j] = from_float<bf16_t>(acc * gv);
+  } else {
+    for (int j = tid; j < dv; j += 256) {
+      const bf16_t* w = W_uv + ((size_t)head * dv + j) * rank;
+      float acc = 0.f;
+      for (int c = 0; c < rank; ++c) acc = fmaf(to_float(w[c]), lat[c], acc);
+      out[unit * dv + j] = from_float<bf16_t>(acc * gv);
+    }
   }
 }
 
