@@ -77,10 +77,16 @@ def configs() -> dict[str, dict]:
         "G": model(180, 64, 3, 1e-5, [
             latent(4, 16, 64, 16, 192, 0.08, 1e4, scaling=(16.0, 64, 8.0, 1.0), mlp=moe(3, 2, 40)),
             latent(1, 32, 16, 48, 48, 0.2, 2e3, mlp=dense(80))]),
+        # head counts that are no power of two over keys that the matrix-core kernels take (64, 32 and 192 elements)
+        "H": model(140, 96, 2, 1e-6, [
+            latent(3, 24, 16, 8, 48, 0.15, 1e4, mlp=dense(64)),
+            latent(5, 8, 8, 24, 24, 0.3, 300.0, scaling=(3.0, 32, 6.0, 1.0), mlp=moe(2, 1, 48)),
+            latent(7, 16, 32, 16, 160, 0.07, 5e3, mlp=dense(64)),
+            attention(6, 2, 32, 32, 0.2, q_temp=(0.2, 10))]),
     }
 
 
-BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16, "F": 16, "G": 16}
+BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16, "F": 16, "G": 16, "H": 64}
 
 
 def wants_of(cfg: dict):
