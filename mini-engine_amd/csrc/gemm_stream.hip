@@ -340,20 +340,31 @@ __global__ __launch_bounds__(256) void gemm_stream_kernel(const bf16_t* __restri
 // for four runs at a time and for one row after the other took a trip to memory for each (a second row cost the kernel
 // 2.3 us, sixteen runs instead of four 0.8). A run beyond the last reads the last one again and counts for nothing; so
 // does a row beyond the last.
-template <int ROWS, int PB>
+// With several residual streams (SMAX > 1; streams.hip) the row that is normed is a weighted sum of the streams, and the
+// pending result rewrites every stream first: new[t] = sum_s mix[s, t] old[s] + out[t] y, u = sum_t in[t] new[t].
+struct StreamArgs {
+  const float* mix_out = nullptr;  // float32 [S * S + S]: mix[from, to], then out[to] (null: nothing is pending)
+  const float* w_in = nullptr;     // float32 [S]: what the coming part reads of each stream
+  size_t stride = 0;               // elements from one stream to the next, in x_in and in x_out
+  int S = 1;
+};
+
+template <int ROWS, int PB, int SMAX = 1>
 struct NormLoads {
-  float4 sv[ROWS], wv, pv[PB][ROWS];
+  float4 sv[SMAX][ROWS], wv, pv[PB][ROWS];
   uint2 dv[ROWS];
 };
 
-template <int ROWS, int PB>
-__device__ __forceinline__ void norm_fetch(NormLoads<ROWS, PB>& ld, const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
+template <int ROWS, int PB, int SMAX = 1>
+__device__ __forceinline__ void norm_fetch(NormLoads<ROWS, PB, SMAX>& ld, const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
                                            const float* __restrict__ parts, int num_parts, size_t part_stride,
-                                           const float* __restrict__ w_norm, int m0, int M, int K, int v) {
+                                           const float* __restrict__ w_norm, int m0, int M, int K, int v, const StreamArgs& st = StreamArgs()) {
 #pragma unroll
   for (int j = 0; j < ROWS; ++j) {
     const size_t at = (size_t)min(m0 + j, M - 1) * K + 4 * v;
-    ld.sv[j] = *reinterpret_cast<const float4*>(x_in + at);
+#pragma unroll
+    for (int s = 0; s < SMAX; ++s)
+      ld.sv[s][j] = s == 0 || s < st.S ? *reinterpret_cast<const float4*>(x_in + (size_t)s * st.stride + at) : make_float4(0.f, 0.f, 0.f, 0.f);
     ld.dv[j] = make_uint2(0, 0);
     if (delta) ld.dv[j] = *reinterpret_cast<const uint2*>(delta + at);
   }
@@ -370,16 +381,16 @@ __device__ __forceinline__ void norm_fetch(NormLoads<ROWS, PB>& ld, const float*
 
 // The rows' sums from what norm_fetch brought (and from the runs beyond the first PB), their squares into ss, the sums
 // themselves to x_out if given, bf16(s * w_norm) into xn.
-template <int ROWS, int PB>
-__device__ __forceinline__ void norm_finish(const NormLoads<ROWS, PB>& ld, const bf16_t* __restrict__ delta,
+template <int ROWS, int PB, int SMAX = 1>
+__device__ __forceinline__ void norm_finish(const NormLoads<ROWS, PB, SMAX>& ld, const bf16_t* __restrict__ delta,
                                             const float* __restrict__ parts, int num_parts, size_t part_stride,
                                             float* __restrict__ x_out, uint16_t* xn, float (&ss)[ROWS], int m0, int M, int K, int krow,
-                                            int v) {
+                                            int v, const StreamArgs& st = StreamArgs()) {
 #pragma unroll
   for (int j = 0; j < ROWS; ++j) {
     if (m0 + j >= M) break;
     const size_t at = (size_t)(m0 + j) * K + 4 * v;
-    float4 t = ld.sv[j];
+    float4 t = SMAX == 1 ? ld.sv[0][j] : make_float4(0.f, 0.f, 0.f, 0.f);  // (several streams: t is the pending result alone)
     if (delta) {
       t.x += __uint_as_float(ld.dv[j].x << 16), t.y += __uint_as_float(ld.dv[j].x & 0xffff0000u);
       t.z += __uint_as_float(ld.dv[j].y << 16), t.w += __uint_as_float(ld.dv[j].y & 0xffff0000u);
@@ -397,7 +408,30 @@ __device__ __forceinline__ void norm_finish(const NormLoads<ROWS, PB>& ld, const
       }
       t.x += d.x, t.y += d.y, t.z += d.z, t.w += d.w;
     }
-    if (x_out) *reinterpret_cast<float4*>(x_out + at) = t;
+    if constexpr (SMAX > 1) {
+      const float4 y = t;
+      t = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int to = 0; to < SMAX; ++to) {
+        if (to >= st.S) break;
+        float4 nv = ld.sv[to][j];
+        if (st.mix_out) {
+          const float o = st.mix_out[st.S * st.S + to];
+          nv = make_float4(o * y.x, o * y.y, o * y.z, o * y.w);
+#pragma unroll
+          for (int from = 0; from < SMAX; ++from) {
+            if (from >= st.S) break;
+            const float mx = st.mix_out[from * st.S + to];
+            nv.x = fmaf(mx, ld.sv[from][j].x, nv.x), nv.y = fmaf(mx, ld.sv[from][j].y, nv.y);
+            nv.z = fmaf(mx, ld.sv[from][j].z, nv.z), nv.w = fmaf(mx, ld.sv[from][j].w, nv.w);
+          }
+          if (x_out) *reinterpret_cast<float4*>(x_out + (size_t)to * st.stride + at) = nv;
+        }
+        const float wi = st.w_in ? st.w_in[to] : 1.f;
+        t.x = fmaf(wi, nv.x, t.x), t.y = fmaf(wi, nv.y, t.y), t.z = fmaf(wi, nv.z, t.z), t.w = fmaf(wi, nv.w, t.w);
+      }
+    } else if (x_out)
+      *reinterpret_cast<float4*>(x_out + at) = t;
     ss[j] = fmaf(t.x, t.x, ss[j]), ss[j] = fmaf(t.y, t.y, ss[j]), ss[j] = fmaf(t.z, t.z, ss[j]), ss[j] = fmaf(t.w, t.w, ss[j]);
     uint2 packed;
     packed.x = (uint32_t)f32_to_bf16_bits(t.x * ld.wv.x) | ((uint32_t)f32_to_bf16_bits(t.y * ld.wv.y) << 16);
@@ -414,12 +448,12 @@ __device__ __forceinline__ void norm_finish(const NormLoads<ROWS, PB>& ld, const
 // rsqrt(mean(s^2) + eps) at the end (a row's scale is a common factor of its products). Block 0 writes s to
 // x_out, which must not alias x_in: the other blocks still read it. Every block reads all of x_in and the partial
 // sums, so this is for a row or two; no runs of k across blocks.
-template <int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int ROWS, int PB>
+template <int WN, int WK, bool SWIGLU, typename OutT, int STAGES, int ROWS, int PB, int SMAX = 1>
 __device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
                                                       const float* __restrict__ parts, int num_parts, size_t part_stride,
                                                       const float* __restrict__ w_norm, float eps, float* __restrict__ x_out,
                                                       const bf16_t* __restrict__ W, OutT* __restrict__ C, int M, int N, int K,
-                                                      int gate, ColumnDeal deal) {
+                                                      int gate, ColumnDeal deal, const StreamArgs& st = StreamArgs()) {
   static_assert(WN * WK == 4, "four waves per block");
   constexpr int KC = kStepK / WK, CH = KC / 32, ACCS = SWIGLU ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char norm_lds[];
@@ -459,8 +493,8 @@ __device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ 
   // ---- the prologue: every row's sum, its squares, and bf16(s * w_norm) into LDS. What the thread's first elements need
   // is asked for before the weights.
   float* const x_to = blockIdx.x == 0 && (delta != nullptr || parts != nullptr) ? x_out : nullptr;
-  NormLoads<ROWS, PB> ld;
-  norm_fetch<ROWS, PB>(ld, x_in, delta, parts, num_parts, part_stride, w_norm, 0, M, K, min((int)threadIdx.x, K / 4 - 1));
+  NormLoads<ROWS, PB, SMAX> ld;
+  norm_fetch<ROWS, PB, SMAX>(ld, x_in, delta, parts, num_parts, part_stride, w_norm, 0, M, K, min((int)threadIdx.x, K / 4 - 1), st);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int p = 0; p < STAGES; ++p) {
@@ -473,9 +507,9 @@ __device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ 
 #pragma unroll
     for (int j = 0; j < ROWS; ++j) ss[j] = 0.f;
     for (int v = threadIdx.x; v < K / 4; v += 256) {
-      if (!fetched) norm_fetch<ROWS, PB>(ld, x_in, delta, parts, num_parts, part_stride, w_norm, m0, M, K, v);
+      if (!fetched) norm_fetch<ROWS, PB, SMAX>(ld, x_in, delta, parts, num_parts, part_stride, w_norm, m0, M, K, v, st);
       fetched = false;
-      norm_finish<ROWS, PB>(ld, delta, parts, num_parts, part_stride, x_to, xn, ss, m0, M, K, krow, v);
+      norm_finish<ROWS, PB, SMAX>(ld, delta, parts, num_parts, part_stride, x_to, xn, ss, m0, M, K, krow, v, st);
     }
 #pragma unroll
     for (int j = 0; j < ROWS; ++j) {
@@ -560,6 +594,23 @@ __device__ __forceinline__ void gemm_stream_norm_body(const float* __restrict__ 
     for (int j = 0; j < 4; ++j)
       if (nb + j < N) dst[j] = from_float<OutT>(y[j]);
   }
+}
+
+// The same kernel over several residual streams (up to four): the prologue rewrites the streams by the pending result and
+// norms what the coming part reads of them; block 0 writes the new streams to x_out.
+template <int WN, int WK, bool SWIGLU, typename OutT, int STAGES>
+__global__ __launch_bounds__(256) void gemm_stream_norm_streams_kernel(const float* __restrict__ x_in, const bf16_t* __restrict__ delta,
+                                                                       const float* __restrict__ parts, int num_parts,
+                                                                       size_t part_stride, const float* __restrict__ w_norm, float eps,
+                                                                       float* __restrict__ x_out, const bf16_t* __restrict__ W,
+                                                                       OutT* __restrict__ C, int M, int N, int K, int gate,
+                                                                       ColumnDeal deal, StreamArgs st) {
+  if (M == 1)
+    gemm_stream_norm_body<WN, WK, SWIGLU, OutT, STAGES, 1, 8, 4>(x_in, delta, parts, num_parts, part_stride, w_norm, eps, x_out, W, C, M,
+                                                                 N, K, gate, deal, st);
+  else
+    gemm_stream_norm_body<WN, WK, SWIGLU, OutT, STAGES, 2, 4, 4>(x_in, delta, parts, num_parts, part_stride, w_norm, eps, x_out, W, C, M,
+                                                                 N, K, gate, deal, st);
 }
 
 // One row: up to sixteen runs of partial sums in the prologue's first request; more rows: two at a time, eight runs.
@@ -805,7 +856,7 @@ namespace {
 template <bool SWIGLU, typename OutT>
 int launch_norm(StreamPlan plan, const float* x_in, const bf16_t* delta, const float* parts, int num_parts, size_t part_stride,
                 const float* w_norm, float eps, float* x_out, const bf16_t* W, OutT* C, int M, int N, int K, int gate,
-                hipStream_t stream) {
+                hipStream_t stream, const StreamArgs* st = nullptr) {
   const dim3 grid(plan.grid);
   const int wn = plan.wn, wk = 4 / wn;
   const size_t rows_bytes = (((size_t)M * (K + 8) * 2 + 15) & ~(size_t)15) + (size_t)M * 4 * sizeof(float);
@@ -813,9 +864,16 @@ int launch_norm(StreamPlan plan, const float* x_in, const bf16_t* delta, const f
   const size_t lds = std::max(rows_bytes, sums_bytes);
   if (lds > 48 * 1024) return me_fail("me_gemm_bf16_stream_norm: %d rows of %d do not fit the block's memory", M, K);
 #define ME_NORM_LAUNCH(WN, WK, STAGES)                                                                                   \
-  gemm_stream_norm_kernel<WN, WK, SWIGLU, OutT, STAGES><<<grid, 256, lds, stream>>>(x_in, delta, parts, num_parts, part_stride, \
-                                                                                    w_norm, eps, x_out, W, C, M, N, K, gate, \
-                                                                                    deal_of(N, plan.grid, K % 2048 == 0))
+  do {                                                                                                                   \
+    if (st)                                                                                                              \
+      gemm_stream_norm_streams_kernel<WN, WK, SWIGLU, OutT, STAGES><<<grid, 256, lds, stream>>>(                         \
+          x_in, delta, parts, num_parts, part_stride, w_norm, eps, x_out, W, C, M, N, K, gate,                           \
+          deal_of(N, plan.grid, K % 2048 == 0), *st);                                                                    \
+    else                                                                                                                 \
+      gemm_stream_norm_kernel<WN, WK, SWIGLU, OutT, STAGES><<<grid, 256, lds, stream>>>(                                 \
+          x_in, delta, parts, num_parts, part_stride, w_norm, eps, x_out, W, C, M, N, K, gate,                           \
+          deal_of(N, plan.grid, K % 2048 == 0));                                                                         \
+  } while (0)
   if (wn == 4)
     ME_NORM_LAUNCH(4, 1, (SWIGLU ? 2 : 3));
   else if (wn == 2)
@@ -837,10 +895,42 @@ extern "C" int me_gemm_bf16_stream_norm_fits(int M, int K) {
 // delta), with the gate as in me_gemm_bf16_stream. x_in float32 [M, K]; the delta is `delta` (bfloat16 [M, K]) or `parts`
 // (float32 [num_parts] of [M, K], part_stride elements apart, added in their order) or neither; with a delta the sum
 // is written to x_out (float32 [M, K], not aliasing x_in). w_norm float32 [K].
+static int stream_norm_common(const float* x_in, const void* delta, const float* parts, int num_parts, long long part_stride,
+                              const float* w_norm, float eps, float* x_out, const void* W, void* C, int M, int N, int K, int swiglu,
+                              int out_dtype, int compute_units, hipStream_t stream, const StreamArgs* st);
+
 extern "C" int me_gemm_bf16_stream_norm(const float* x_in, const void* delta, const float* parts, int num_parts,
                                         long long part_stride, const float* w_norm, float eps, float* x_out, const void* W,
                                         void* C, int M, int N, int K, int swiglu, int out_dtype, int compute_units,
                                         hipStream_t stream) {
+  return stream_norm_common(x_in, delta, parts, num_parts, part_stride, w_norm, eps, x_out, W, C, M, N, K, swiglu, out_dtype,
+                            compute_units, stream, nullptr);
+}
+
+// The same over `streams` residual streams (up to 4; xs float32 [streams, M, K], stream_stride elements apart, as is
+// xs_out): C[M, N] = rmsnorm(sum_t in[t] new[t]) * w_norm . W^T with new[t] = sum_s mix[s, t] xs[s] + out[t] (delta or partial
+// sums) where a result is pending (mix_out float32 [S * S + S]; then the new streams go to xs_out), else new = xs.
+extern "C" int me_gemm_bf16_stream_norm_streams(const float* xs, long long stream_stride, int streams, const void* delta,
+                                                const float* parts, int num_parts, long long part_stride, const float* mix_out,
+                                                const float* w_in, const float* w_norm, float eps, float* xs_out, const void* W,
+                                                void* C, int M, int N, int K, int swiglu, int out_dtype, int compute_units,
+                                                hipStream_t stream) {
+  if (streams < 1 || streams > 4) return me_fail("me_gemm_bf16_stream_norm_streams: %d streams, 1 to 4 are taken", streams);
+  if (stream_stride < (long long)M * K || stream_stride % 4) return me_fail("me_gemm_bf16_stream_norm_streams: streams %lld elements apart", stream_stride);
+  if ((delta || parts) && !mix_out) return me_fail("me_gemm_bf16_stream_norm_streams: a pending result needs its coefficients");
+  if (!w_in) return me_fail("me_gemm_bf16_stream_norm_streams: what the part reads of the streams is missing");
+  StreamArgs st;
+  st.mix_out = (delta || parts) ? mix_out : nullptr;
+  st.w_in = w_in;
+  st.stride = (size_t)stream_stride;
+  st.S = streams;
+  return stream_norm_common(xs, delta, parts, num_parts, part_stride, w_norm, eps, xs_out, W, C, M, N, K, swiglu, out_dtype,
+                            compute_units, stream, &st);
+}
+
+static int stream_norm_common(const float* x_in, const void* delta, const float* parts, int num_parts, long long part_stride,
+                              const float* w_norm, float eps, float* x_out, const void* W, void* C, int M, int N, int K, int swiglu,
+                              int out_dtype, int compute_units, hipStream_t stream, const StreamArgs* st) {
   if (M <= 0 || N <= 0) return 0;
   if (swiglu < ME_GATE_NONE || swiglu > ME_GATE_GELU_TANH) return me_fail("me_gemm_bf16_stream_norm: unknown gate activation %d", swiglu);
   if (!me_gemm_bf16_stream_norm_fits(M, K)) return me_fail("me_gemm_bf16_stream_norm: M=%d rows of K=%d are not taken", M, K);
@@ -861,8 +951,8 @@ extern "C" int me_gemm_bf16_stream_norm(const float* x_in, const void* delta, co
   const bf16_t *d = (const bf16_t*)delta, *w = (const bf16_t*)W;
   const size_t stride = parts ? (size_t)part_stride : 0;
   if (swiglu)
-    return launch_norm<true, bf16_t>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, swiglu, stream);
+    return launch_norm<true, bf16_t>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, swiglu, stream, st);
   if (out_dtype == ME_F32)
-    return launch_norm<false, float>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (float*)C, M, N, K, 0, stream);
-  return launch_norm<false, bf16_t>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, 0, stream);
+    return launch_norm<false, float>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (float*)C, M, N, K, 0, stream, st);
+  return launch_norm<false, bf16_t>(plan, x_in, d, parts, num_parts, stride, w_norm, eps, x_out, w, (bf16_t*)C, M, N, K, 0, stream, st);
 }

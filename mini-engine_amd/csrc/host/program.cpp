@@ -177,7 +177,7 @@ class Run {
       : prog_(prog), values_(values), s_(s), arena_(arena), fed_tokens_(fed_tokens), stream_(stream), dtype_(prog.dtype()),
         elem_(prog.dtype() == kF32 ? 4 : 2), t_(s.lay.tokens), h_(prog.hidden()), streams_(streams_of(prog.ops())) {
     x_ = (float*)arena_.take((size_t)streams_ * t_ * h_ * 4);  // (several streams: [streams, tokens, hidden], x_ is the first)
-    spare_ = (float*)arena_.take((size_t)t_ * h_ * 4);
+    spare_ = (float*)arena_.take((size_t)streams_ * t_ * h_ * 4);
     normed_ = arena_.take((size_t)t_ * h_ * elem_);
     for (const Value& v : values) bufs_.push_back(arena_.take((size_t)t_ * v.cols * v.elem));
   }
@@ -278,6 +278,9 @@ class Run {
         break;
       case kOpStreamHead:
         stream_head(op);
+        break;
+      case kOpStreamNormLinear:
+        stream_norm_linear(op);
         break;
       case kOpLatentAttention:
         latent_attention(op);
@@ -649,6 +652,37 @@ class Run {
     if (op.kind != kOpStreamHead) release_parts();  // (the head's buffers lie behind waiting partial sums)
   }
 
+  // The rewrite of the streams, the norm and the product behind it: for a row or two of a bfloat16 step all in the
+  // product's kernel (every block rewrites and norms the rows while its first weights are on their way; block 0 writes the
+  // new streams to the second set of buffers); else the norm as a kernel of its own, then the product.
+  void stream_norm_linear(const Op& op) {
+    const int rows_of_w = (int)op.i[0], k = (int)op.i[1], gated = (int)op.i[2];
+    if (k != h_) throw Error(kBadValue, "a product behind a norm reads the hidden size");
+    if (!spread_) throw Error(kBroken, "a norm over several streams before the streams begin");
+    if (held_.any() || pending_.carried()) throw Error(kBroken, "several streams take one pending result at a time");
+    if (pending_.any() && !op.p[2]) throw Error(kBroken, "a result is pending and nothing says how it rewrites the streams");
+    if (pending_.any() && pending_.scale != 1.f) throw Error(kBroken, "a result of several streams is not scaled");
+    const int n = gated ? rows_of_w / 2 : rows_of_w;
+    const int pending = pending_.parts ? kPendingParts : pending_.delta ? kPendingTensor : kPendingNone;
+    if (streams_ <= 4 && choose_norm_fusion(dtype_, t_, rows_of_w, k, pending, compute_units(), true) == kNormInStream) {
+      const bool adds = pending_.any();
+      ok(me_gemm_bf16_stream_norm_streams(x_, (long long)t_ * h_, streams_, pending_.delta, pending_.parts, pending_.num_parts,
+                                          pending_.stride, (const float*)op.p[2], (const float*)op.p[3], (const float*)op.p[0], op.f[0],
+                                          adds ? spare_ : nullptr, op.p[1], bufs_[op.out], t_, n, k, gated, dtype_, compute_units(),
+                                          stream_));
+      if (adds) std::swap(x_, spare_);
+      pending_ = Pending();
+      release_parts();
+      return;
+    }
+    ok(me_streams_norm(x_, (long long)t_ * h_, streams_, pending_.delta, pending_.parts, pending_.num_parts, pending_.stride,
+                       pending_.any() ? (const float*)op.p[2] : nullptr, (const float*)op.p[3], (const float*)op.p[0], normed_, nullptr, t_,
+                       h_, op.f[0], 1, dtype_, stream_));
+    pending_ = Pending();
+    release_parts();
+    product(normed_, op.p[1], rows_of_w, k, gated, dtype_, bufs_[op.out]);
+  }
+
   void stream_head(const Op& op) {
     const int rows = s_.lay.rows;
     result_.rows = rows;
@@ -856,12 +890,12 @@ std::vector<std::vector<int>> Program::prefill_geometries() const {
 size_t Program::arena_need(int64_t tokens, int64_t items, int64_t rows, int64_t max_ctx) const {
   const size_t elem = dtype_ == kF32 ? 4 : 2;
   const size_t pad = 256;
-  size_t fixed = (1 + (size_t)streams_of(ops_)) * ((size_t)tokens * hidden_ * 4 + pad) + (size_t)tokens * hidden_ * elem + pad;
+  size_t fixed = 2 * (size_t)streams_of(ops_) * ((size_t)tokens * hidden_ * 4 + pad) + (size_t)tokens * hidden_ * elem + pad;
   for (const Value& v : values_) fixed += (size_t)tokens * v.cols * v.elem + pad;
   size_t scratch = 0;
   for (const Op& op : ops_) {
     size_t need = 0;
-    if (op.kind == kOpNormLinear || op.kind == kOpLinear) need = (size_t)tokens * op.i[0] * 4 + pad;
+    if (op.kind == kOpNormLinear || op.kind == kOpLinear || op.kind == kOpStreamNormLinear) need = (size_t)tokens * op.i[0] * 4 + pad;
     if (op.kind == kOpLinearDelta)  // up to 16 partial sums of up to 64 rows, or one float32 result of all rows
       need = std::max<size_t>((size_t)kMaxRuns * std::min<int64_t>(tokens, kSmallMaxRows), (size_t)tokens) * op.i[0] * 4 + pad;
     if (op.kind == kOpDecayState)

@@ -66,6 +66,9 @@ enum OpKind {
   kOpRoutedFF = 18,   // in: normed activations; p0 router W float32 [E, hidden], p1 experts' gate and up rows [E, 2 ff, hidden],
                       // p2 experts' down rows [E, hidden, ff]; i0 E, i1 experts a token, i2 ff, i3 code of the activation
                       // -> pending (partial sums, one per expert of a token)
+  kOpStreamNormLinear = 19,  // kOpStreamNorm and the product behind it: p0 norm weight, f0 eps, p1 W [rows, hidden], p2 how the pending
+                      // result rewrites the streams (or null), p3 what the product's part reads of each stream; i0 rows of W, i1 K,
+                      // i2 gated; pending + streams -> streams, out
 };
 // kOpLinearDelta i2: the result stays pending whatever the step's size (no product adds itself to the stream).
 // kOpAttention beyond i12: i13 every (0: none) and f2 coef of a temperature on the queries, 1 + coef * ln(floor((position + 1) / every)

@@ -149,6 +149,10 @@ int me_gemm_bf16_stream_norm_fits(int M, int K);
 int me_gemm_bf16_stream_norm(const float* x_in, const void* delta, const float* parts, int num_parts, long long part_stride,
                              const float* w_norm, float eps, float* x_out, const void* W, void* C, int M, int N, int K,
                              int swiglu, int out_dtype, int compute_units, hipStream_t stream);
+int me_gemm_bf16_stream_norm_streams(const float* xs, long long stream_stride, int streams, const void* delta, const float* parts,
+                                     int num_parts, long long part_stride, const float* mix_out, const float* w_in, const float* w_norm,
+                                     float eps, float* xs_out, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype,
+                                     int compute_units, hipStream_t stream);
 int me_gemm_bf16_tiled(const void* X, const void* W, void* C, int M, int N, int K, int swiglu, int out_dtype, int shape,
                        hipStream_t stream);
 int me_gemm_bf16_library(const void* X, const void* W, void* C, int M, int N, int K, int out_dtype, hipStream_t stream);

@@ -29,7 +29,7 @@ _vp, _i64, _i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
 _declared = False
 
 (EMBED, NORM_LINEAR, NORM, LINEAR, LINEAR_DELTA, DELTA, ATTENTION, HEAD, SAMPLE, ADD, CALL, HEAD_ROWS, DECAY_STATE, HOLD, STREAMS,
- STREAM_NORM, STREAM_HEAD, LATENT_ATTENTION, ROUTED_FF) = range(19)
+ STREAM_NORM, STREAM_HEAD, LATENT_ATTENTION, ROUTED_FF, STREAM_NORM_LINEAR) = range(20)
 OP_PTRS, OP_INTS, OP_FLOATS = 8, 16, 4  # csrc/host/program.h: kOpPtrs, kOpInts, kOpFloats
 MAX_STREAMS = 8  # csrc/streams.hip: ME_MAX_STREAMS
 _RAISES = {1: ValueError, 2: RuntimeError, 3: AssertionError}
@@ -134,6 +134,27 @@ class CalledNorm:
             p, norm = self.program, self.norm
             p.add()
             self._value = p.call(lambda frame: frame.output.copy_(norm.forward(frame.x)), out_cols=p.hidden)
+            self.used = True
+        return self._value
+
+
+class StreamNormed:
+    """As :class:`Normed`, over several residual streams: the pending rewrite of the streams, the read of the coming part's
+    input and its norm, not yet written into the program. The part's first product takes it as its input (the program then
+    puts all of it into that product's kernel where the step is small enough); ``value()`` gives the normed input as a value
+    of its own."""
+
+    def __init__(self, program: "StepProgram", weight: torch.Tensor, eps: float, reads: torch.Tensor, rewrite: torch.Tensor | None):
+        self.program, self.weight, self.eps, self.reads, self.rewrite = program, weight, float(eps), reads, rewrite
+        self.used = False
+        self._value: int | None = None
+
+    def value(self) -> int:
+        if self._value is None:
+            p = self.program
+            self._value = p.take(p.hidden, p.elem)
+            p.op(STREAM_NORM, out=self._value, ptrs=[self.weight, self.rewrite, self.reads], floats=[self.eps])
+            p.pending_consumed()
             self.used = True
         return self._value
 
@@ -251,7 +272,14 @@ class StepProgram:
             x.used = True
             self.pending_consumed()
             return out
-        src = x.value() if isinstance(x, (Normed, CalledNorm)) else x
+        if isinstance(x, StreamNormed) and x._value is None:
+            if k != self.hidden:
+                raise ValueError("a product behind the norm reads the hidden size")
+            self.op(STREAM_NORM_LINEAR, out=out, ptrs=[x.weight, weight, x.rewrite, x.reads], ints=[rows, k, gate], floats=[x.eps])
+            x.used = True
+            self.pending_consumed()
+            return out
+        src = x.value() if isinstance(x, (Normed, CalledNorm, StreamNormed)) else x
         if self._value_kinds[src][0] != k:
             raise ValueError(f"the weight reads {k} columns, the value has {self._value_kinds[src][0]}")
         self.op(LINEAR, in_=src, out=out, ptrs=[None, weight], ints=[rows, k, gate])
@@ -370,19 +398,17 @@ class StepProgram:
         self.op(STREAMS, ints=[streams])
         self.num_streams = int(streams)
 
-    def stream_normed(self, norm, reads: torch.Tensor) -> int:
-        """The input of the coming part as a value: the pending result rewrites the streams (by what :meth:`rewrites_streams`
-        said of it), ``sum_s reads[s] x_s`` is normed by ``norm`` (RMS-shaped)."""
+    def stream_normed(self, norm, reads: torch.Tensor) -> StreamNormed:
+        """The input of the coming part, not yet written: the pending result rewrites the streams (by what
+        :meth:`rewrites_streams` said of it), ``sum_s reads[s] x_s`` is normed by ``norm`` (RMS-shaped). The part's first product
+        takes it (:meth:`linear`), or its ``value()`` does."""
         weight, eps = norm.as_fused()
         if getattr(norm, "groups", 1) != 1:
             raise ValueError("the norm over several streams is not cut into groups")
         self._want(weight, torch.float32, (self.hidden,), "norm weight")
         self._want(reads, torch.float32, (self.num_streams,), "what a part reads of the streams")
-        out = self.take(self.hidden, self.elem)
-        self.op(STREAM_NORM, out=out, ptrs=[weight, self._stream_rewrite, reads], floats=[eps])
-        self._stream_rewrite = None
-        self.pending_consumed()
-        return out
+        rewrite, self._stream_rewrite = self._stream_rewrite, None
+        return StreamNormed(self, weight, eps, reads, rewrite)
 
     def rewrites_streams(self, mix_out: torch.Tensor) -> None:
         """The result that is pending now rewrites the streams by ``mix_out`` float32 ``[S * S + S]``: ``mix[from, to]``, then

@@ -1320,3 +1320,36 @@ def routed_ff(h: torch.Tensor, router: torch.Tensor, gate_up: torch.Tensor, down
     check(lib().me_routed_ff(_p(h), _p(router), _p(gate_up), _p(down), _p(parts), _p(ws), _i(t), _i(hidden), _i(e), _i(top_k),
                              _i(two_ff // 2), _i(gate_code(activation)), _i(_code(h.dtype)), _stream()))
     return PartialSums(parts)
+
+
+def gemm_bf16_stream_norm_streams(xs: torch.Tensor, delta, rewrite: torch.Tensor | None, reads: torch.Tensor, norm_weight: torch.Tensor,
+                                  eps: float, weight: torch.Tensor, gated: "bool | str" = False,
+                                  out_dtype: torch.dtype = torch.bfloat16) -> tuple[torch.Tensor, torch.Tensor]:
+    """:func:`streams_norm` and the bfloat16 product behind it in one kernel, for a row or two: ``xs`` float32 ``[S, M, K]`` (up to
+    four streams) is rewritten by the pending result ``delta`` (bfloat16 ``[M, K]``, :class:`PartialSums` or None) and
+    ``rewrite``, ``sum_s reads[s] xs[s]`` is normed by ``norm_weight`` and multiplied by ``weight`` ``[N (2 N gated), K]``.
+    Returns (the product ``[M, N]``, the streams as they are afterwards: a new tensor when a result was pending, else ``xs``)."""
+    _want(xs, "xs", torch.float32, (None, None, None))
+    s, m, k = xs.shape
+    rows = weight.shape[0]
+    _want(weight, "weight", torch.bfloat16, (rows, k))
+    _want(norm_weight, "norm weight", torch.float32, (k,))
+    _want(reads, "reads", torch.float32, (s,))
+    parts = delta if isinstance(delta, PartialSums) else None
+    tensor = None if parts is not None else delta
+    if tensor is not None:
+        _want(tensor, "delta", torch.bfloat16, (m, k))
+    if parts is not None:
+        _want(parts.parts, "partial sums", torch.float32, (None, m, k))
+    if rewrite is not None:
+        _want(rewrite, "rewrite", torch.float32, (s * s + s,))
+    gate = gate_code(gated)
+    n = rows // 2 if gate else rows
+    out = torch.empty((m, n), dtype=out_dtype, device=xs.device)
+    pending = delta is not None
+    new = torch.empty_like(xs) if pending else xs
+    check(lib().me_gemm_bf16_stream_norm_streams(
+        _p(xs), _i64(m * k), _i(s), _p(tensor), _p(None if parts is None else parts.parts), _i(0 if parts is None else parts.parts.shape[0]),
+        _i64(m * k), _p(rewrite), _p(reads), _p(norm_weight), _f(eps), _p(new if pending else None), _p(weight), _p(out), _i(m), _i(n),
+        _i(k), _i(gate), _i(_code(out_dtype)), _i(compute_units(xs.device)), _stream()))
+    return out, new

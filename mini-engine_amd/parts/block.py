@@ -181,7 +181,9 @@ class HyperConnectionBlock:
                     out = part.emit(program, h, *extra)
                 else:
                     out = program.call(lambda frame, part=part, extra=extra: frame.write(part.forward(frame.input, frame.batch, *extra)),
-                                       in_=h, out_cols=program.hidden)
+                                       in_=h.value(), out_cols=program.hidden)
+                if not h.used:  # the part never looked at its input: the streams' rewrite still has to happen
+                    h.value()
                 if out is not None:
                     program.delta(out)
                 program.rewrites_streams(self.rewrites[tie.prefix])

@@ -167,7 +167,7 @@ def rows_that_bear_rounding(cfg: dict, weights: dict, tokens: list[int], share: 
     return (exact - rounded).abs().amax(-1) < share * exact.abs().amax(-1)
 
 
-def rows_before_a_close_call(cfg: dict, weights: dict, tokens: list[int], share: float = 0.005) -> int:
+def rows_before_a_close_call(cfg: dict, weights: dict, tokens: list[int], share: float = 0.01) -> int:
     """How many leading positions of a sequence no router decides by less than ``share`` of its largest logit: up to there
     a rounding of the activations cannot change which experts a token uses (nor, through the keys and values that the
     token leaves, what later tokens read)."""

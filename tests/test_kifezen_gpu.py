@@ -60,6 +60,38 @@ def test_streams_are_rewritten_read_and_normed(streams, dim, dtype):
     assert all(torch.equal(spread[s].cpu(), xs[0]) for s in range(streams))
 
 
+@pytest.mark.parametrize("streams,rows,k,n,gated", [(1, 1, 128, 96, False), (2, 1, 1024, 256, True), (2, 2, 256, 520, False),
+                                                     (3, 1, 96, 64, True), (4, 2, 512, 128, False)])
+def test_the_product_that_rewrites_reads_and_norms_the_streams_itself(streams, rows, k, n, gated):
+    """The norm's kernel and the product behind it as one kernel (a row or two, bfloat16): a tensor pending, partial sums
+    pending, nothing pending."""
+    from mini_engine_amd.ops import kernels as K
+
+    g = torch.Generator().manual_seed(streams * 100 + k)
+    xs = torch.randn(streams, rows, k, generator=g)
+    mix, out = torch.eye(streams) + 0.3 * torch.randn(streams, streams, generator=g), 1 + 0.3 * torch.randn(streams, generator=g)
+    reads = torch.randn(streams, generator=g)
+    w_norm = 0.2 * torch.randn(k, generator=g)
+    weight = (0.1 * torch.randn(2 * n if gated else n, k, generator=g)).to(torch.bfloat16)
+    rewrite = torch.cat((mix.reshape(-1), out)).cuda()
+    y = torch.randn(rows, k, generator=g).to(torch.bfloat16)
+    parts = torch.randn(6, rows, k, generator=g)
+
+    def want_of(new):
+        h = plain.offset_norm(plain.streams_read(new, reads.to(F64)), w_norm.to(F64), 1e-5)
+        z = h @ weight.to(F64).T
+        return plain.silu(z[:, :n]) * z[:, n:] if gated else z
+
+    for pending, y64 in ((y.cuda(), y.to(F64)), (K.PartialSums(parts.cuda()), parts.to(F64).sum(0)), (None, None)):
+        dev = xs.cuda()
+        got, new_dev = K.gemm_bf16_stream_norm_streams(dev, pending, rewrite if pending is not None else None, reads.cuda(),
+                                                      (1.0 + w_norm).cuda(), 1e-5, weight.cuda(), gated="silu" if gated else False)
+        new = xs.to(F64) if y64 is None else plain.streams_write(xs.to(F64), y64, mix.to(F64), out.to(F64))
+        assert torch.equal(dev.cpu(), xs)  # the streams it read are left as they were
+        assert rel_err(new_dev.reshape(streams * rows, k), new.reshape(streams * rows, k)) < 1e-6
+        assert rel_err(got, want_of(new)) < TOL[torch.bfloat16]
+
+
 # ---------------------------------------------------------------------------------------- attention
 def shuffled_table(items_len: list[int], bs: int, seed: int):
     """A block table whose pages lie in no order (as pages that were freed and taken again do), and the pool's size."""
@@ -311,7 +343,7 @@ def test_every_way_of_cutting_gives_the_plain_logits(folders, name, dtype):
         for rid, t in reqs.items():
             keep[rid] = kh.rows_that_bear_rounding(cfg, weights, t)
             keep[rid][kh.rows_before_a_close_call(cfg, weights, t):] = False
-    assert sum(int(k.sum()) for k in keep.values()) > 0.15 * sum(len(t) for t in reqs.values())
+    assert sum(int(k.sum()) for k in keep.values()) > 0.05 * sum(len(t) for t in reqs.values())  # (float32 compares every row)
     bs = kh.BLOCK_SIZES[name]
     biggest = max(th.round_up(len(t)) for t in reqs.values())
     for build, max_tokens, live in ((th.whole, biggest, 4), (lambda r: th.tail_one_by_one(r, tail=40), biggest, 4),
