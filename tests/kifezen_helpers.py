@@ -83,10 +83,15 @@ def configs() -> dict[str, dict]:
             latent(5, 8, 8, 24, 24, 0.3, 300.0, scaling=(3.0, 32, 6.0, 1.0), mlp=moe(2, 1, 48)),
             latent(7, 16, 32, 16, 160, 0.07, 5e3, mlp=dense(64)),
             attention(6, 2, 32, 32, 0.2, q_temp=(0.2, 10))]),
+        # sizes that are no multiple of 8 (a width of 100, feed-forwards of 52 and 20, a latent of 30 + 6): every product takes
+        # the kernels that take any size; five streams: more than the product that norms the streams itself takes
+        "I": model(211, 100, 5, 1e-5, [
+            latent(3, 10, 6, 14, 30, 0.25, 1e3, scaling=(2.0, 16, 4.0, 1.0), mlp=moe(5, 2, 20)),
+            attention(5, 1, 12, 20, 0.3, q_temp=(0.6, 3), mlp=dense(52))]),
     }
 
 
-BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16, "F": 16, "G": 16, "H": 64}
+BLOCK_SIZES = {"A": 16, "B": 32, "C": 8, "D": 16, "E": 16, "F": 16, "G": 16, "H": 64, "I": 16}
 
 
 def wants_of(cfg: dict):
